@@ -1,0 +1,39 @@
+"""Tiny configurations and small helpers shared by the tests."""
+
+from __future__ import annotations
+
+import torch
+
+
+def qwen3_config(*, hidden, layers, heads, kv_heads, head_dim, inter, vocab, eps, theta,
+                 tied, max_pos, window=None, layer_types=None):
+    cfg = {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3",
+        "hidden_size": hidden, "num_hidden_layers": layers, "num_attention_heads": heads,
+        "num_key_value_heads": kv_heads, "head_dim": head_dim, "intermediate_size": inter,
+        "vocab_size": vocab, "rms_norm_eps": eps, "rope_theta": theta,
+        "max_position_embeddings": max_pos, "tie_word_embeddings": tied,
+        "hidden_act": "silu", "attention_bias": False, "rope_scaling": None,
+        "sliding_window": window, "use_sliding_window": window is not None,
+    }
+    if layer_types is not None:
+        cfg["layer_types"] = layer_types
+    return cfg
+
+
+# Two configurations that differ in every size and option, plus one with windowed
+# layers.  A and B are the two tiny configurations the benchmark description names.
+TINY_A = qwen3_config(hidden=64, layers=2, heads=4, kv_heads=2, head_dim=16, inter=128,
+                      vocab=256, eps=1e-6, theta=10000.0, tied=True, max_pos=128)
+TINY_B = qwen3_config(hidden=96, layers=3, heads=8, kv_heads=2, head_dim=32, inter=160,
+                      vocab=389, eps=1e-5, theta=1e6, tied=False, max_pos=256)
+TINY_C = qwen3_config(hidden=80, layers=4, heads=6, kv_heads=3, head_dim=48, inter=112,
+                      vocab=301, eps=3e-6, theta=50000.0, tied=False, max_pos=512,
+                      window=24, layer_types=["full_attention", "sliding_attention",
+                                              "sliding_attention", "full_attention"])
+TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 8)}   # cfg, seed, page
+
+
+def random_prompt(length, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (length,), generator=g).tolist()

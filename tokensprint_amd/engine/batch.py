@@ -1,0 +1,150 @@
+"""One step's batch: what every kernel needs to know about the tokens it is given.
+
+The reference flattens a step into input_ids, positions, cu_seqlens_q/k,
+slot_mapping, context_lens, block_tables and seq_need_compute_logits with one Python
+loop per token (engine/generation/model_runner.py:101-168, 64-99).  Here the same
+facts travel as one int32 buffer copied to the device once; the cache slot of a token
+is computed inside the kernels from the block table, so there is no per-token host
+loop for it.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from tokensprint_amd.cache.pages import RequestCache
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens: positions [start, start+len(tokens)), and the
+    offsets among these tokens whose logits are wanted."""
+
+    cache: RequestCache
+    tokens: list[int]
+    start: int
+    want: list[int] = field(default_factory=list)
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    token_ids: torch.Tensor        # int32 [T]
+    positions: torch.Tensor        # int32 [T]
+    entry_of_token: torch.Tensor   # int32 [T]
+    q_start: torch.Tensor          # int32 [B+1]  first flat token of each entry
+    ctx_len: torch.Tensor          # int32 [B]    keys of the entry after this step
+    slot_ids: torch.Tensor         # int32 [B]    state slot of each entry
+    logit_rows: torch.Tensor       # int32 [R]    flat token index of each wanted row
+    tables: list[torch.Tensor]     # per group int32 [B, width_g], -1 = no page
+    # host copies for launch planning
+    q_lens: list[int]
+    starts: list[int]
+    max_q_len: int
+    max_ctx_len: int
+    plans: dict = field(default_factory=dict)   # kernels cache per-step launch plans here
+
+
+def _align(n: int, a: int = 4) -> int:
+    return -(-n // a) * a
+
+
+class BatchBuilder:
+    """Packs a step's description into one pinned buffer and one device copy."""
+
+    def __init__(self, device, num_groups: int, vocab_size: int | None = None,
+                 max_position: int | None = None) -> None:
+        self.device = torch.device(device)
+        self.num_groups = num_groups
+        self.vocab_size = vocab_size
+        self.max_position = max_position
+        self._pinned = None
+
+    def _host_buffer(self, n: int) -> torch.Tensor:
+        if self.device.type != "cuda":
+            return torch.empty(n, dtype=torch.int32)
+        if self._pinned is None or self._pinned.numel() < n:
+            self._pinned = torch.empty(max(n, 1 << 16), dtype=torch.int32, pin_memory=True)
+        return self._pinned[:n]
+
+    def build(self, entries: list[StepEntry], table_width: list[int] | None = None) -> StepBatch:
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        B = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        starts = [e.start for e in entries]
+        if min(q_lens) < 1:
+            raise ValueError("every entry of a step brings at least one token")
+        T = sum(q_lens)
+        for e, n in zip(entries, q_lens):
+            if e.start < 0 or e.start + n > e.cache.num_tokens:
+                raise ValueError(
+                    f"request {e.cache.request_id!r}: tokens at [{e.start}, {e.start + n}) "
+                    f"but its cache covers {e.cache.num_tokens} positions")
+            if self.max_position is not None and e.start + n > self.max_position:
+                raise ValueError(
+                    f"request {e.cache.request_id!r}: position {e.start + n - 1} is beyond "
+                    f"the model's {self.max_position} positions")
+            if any(not 0 <= w < n for w in e.want):
+                raise ValueError(f"request {e.cache.request_id!r}: wanted offsets {e.want} "
+                                 f"outside its {n} tokens")
+        R = sum(len(e.want) for e in entries)
+        widths = []
+        for g in range(self.num_groups):
+            w = max(len(e.cache.tables[g]) for e in entries)
+            if table_width is not None:
+                if w > table_width[g]:
+                    raise ValueError("block table wider than the fixed width")
+                w = table_width[g]
+            widths.append(max(w, 1))
+
+        # layout of the one buffer (every section 16-byte aligned)
+        sizes = [T, T, T, B + 1, B, B, max(R, 1)] + [B * w for w in widths]
+        offs, total = [], 0
+        for s in sizes:
+            offs.append(total)
+            total += _align(s)
+        host = self._host_buffer(total)
+        buf = host.numpy()
+
+        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        if ids.min() < 0 or (self.vocab_size is not None and ids.max() >= self.vocab_size):
+            raise ValueError(f"token id outside [0, {self.vocab_size})")
+        buf[offs[0]:offs[0] + T] = ids
+        qs = np.zeros(B + 1, dtype=np.int64)
+        np.cumsum(q_lens, out=qs[1:])
+        buf[offs[1]:offs[1] + T] = np.concatenate(
+            [np.arange(s, s + n) for s, n in zip(starts, q_lens)])
+        buf[offs[2]:offs[2] + T] = np.repeat(np.arange(B), q_lens)
+        buf[offs[3]:offs[3] + B + 1] = qs
+        buf[offs[4]:offs[4] + B] = [s + n for s, n in zip(starts, q_lens)]
+        buf[offs[5]:offs[5] + B] = [e.cache.slot for e in entries]
+        rows = [int(qs[i]) + w for i, e in enumerate(entries) for w in e.want]
+        buf[offs[6]:offs[6] + R] = rows
+        for g, w in enumerate(widths):
+            tab = np.full((B, w), -1, dtype=np.int32)
+            for i, e in enumerate(entries):
+                t = e.cache.tables[g]
+                tab[i, :len(t)] = t
+            buf[offs[7 + g]:offs[7 + g] + B * w] = tab.reshape(-1)
+
+        dev = host.to(self.device, non_blocking=True) if self.device.type == "cuda" \
+            else host.clone()
+
+        def sec(i, n):
+            return dev[offs[i]:offs[i] + n]
+
+        return StepBatch(
+            num_tokens=T, num_entries=B, num_logit_rows=R,
+            token_ids=sec(0, T), positions=sec(1, T), entry_of_token=sec(2, T),
+            q_start=sec(3, B + 1), ctx_len=sec(4, B), slot_ids=sec(5, B),
+            logit_rows=sec(6, R),
+            tables=[sec(7 + g, B * w).view(B, w) for g, w in enumerate(widths)],
+            q_lens=q_lens, starts=starts, max_q_len=max(q_lens),
+            max_ctx_len=max(s + n for s, n in zip(starts, q_lens)),
+        )

@@ -1,0 +1,94 @@
+"""A model built from a `ModelSpec`: embedding, runs of layers, final norm, head.
+
+Shape of the forward pass is the reference's engine/model.py:58-86 (embedding ->
+every block -> final norm -> gather wanted rows -> output projection), except that
+the rows whose logits are wanted are gathered before the final norm, which is
+row-wise, so only those rows are normalised and projected.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokensprint_amd.models.spec import ModelSpec
+from tokensprint_amd.parts.base import (
+    BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, BuildContext, TensorDecl, build_part,
+)
+from tokensprint_amd.parts.ends import Embedding, Head
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, ctx: BuildContext) -> None:
+        spec.validate()
+        if ctx.width != spec.width:
+            raise ValueError("build context width differs from the model's")
+        self.spec, self.ctx = spec, ctx
+        for name, pspec in spec.positions.items():
+            ctx.positions[name] = build_part(POSITIONS, pspec, ctx)
+        self.embedding = Embedding(dict(spec.embedding.params), ctx)
+        self.blocks = []
+        for layer in spec.layers:
+            if layer.block not in BLOCKS:
+                raise ValueError(f"unknown block kind '{layer.block}'; registered: {sorted(BLOCKS)}")
+            self.blocks.append(BLOCKS[layer.block](
+                build_part(MIXERS, layer.mixer, ctx),
+                build_part(FEED_FORWARDS, layer.feed_forward, ctx),
+                build_part(NORMS, layer.mixer_norm, ctx),
+                build_part(NORMS, layer.ffn_norm, ctx), ctx))
+        self.final_norm = build_part(NORMS, spec.final_norm, ctx)
+        self.head = Head(dict(spec.head.params), ctx)
+        self.order = spec.order
+
+    # ------------------------------------------------------------ weights
+    def parts(self):
+        out = [self.embedding]
+        for block in self.blocks:
+            out.extend(block.parts())
+        out.extend([self.final_norm, self.head])
+        out.extend(self.ctx.positions.values())
+        return out
+
+    def tensor_decls(self) -> dict[str, TensorDecl]:
+        decls: dict[str, TensorDecl] = {}
+        for part in self.parts():
+            for name, decl in part.tensors().items():
+                if name in decls and (decls[name].shape != decl.shape
+                                      or decls[name].role != decl.role):
+                    raise ValueError(f"tensor {name} declared twice with different shapes")
+                # a name needed by any part is not optional
+                if name in decls and not decls[name].optional:
+                    continue
+                decls[name] = decl
+        return decls
+
+    def load_tensors(self, tensors: dict[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.load(tensors.get)
+
+    # ------------------------------------------------------------ caches
+    def cache_needs(self):
+        """Per run: the cache need of its mixer, or None if the run owns no cache."""
+        return [self.blocks[run.layer].mixer.cache_need() if run.cache_of is None else None
+                for run in self.order]
+
+    # ------------------------------------------------------------ step
+    def forward(self, batch, caches) -> torch.Tensor:
+        """Run the batch's tokens; logits float32 [len(batch.logit_rows), vocab].
+
+        `caches[r]` is the cache view owned by run r (None if it owns none).
+        """
+        ops = self.ctx.ops
+        resid = self.embedding.forward(batch.token_ids)
+        delta = None
+        for r, run in enumerate(self.order):
+            owner = r if run.cache_of is None else run.cache_of
+            resid, delta = self.blocks[run.layer].forward(
+                resid, delta, batch, caches[owner], write_cache=run.cache_of is None)
+        if batch.num_logit_rows == 0:
+            return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=resid.device)
+        resid_rows = ops.gather_rows(resid, batch.logit_rows)
+        if delta is None:
+            h = self.final_norm.forward(resid_rows)
+        else:
+            h = self.final_norm.add_forward(resid_rows, ops.gather_rows(delta, batch.logit_rows))
+        return self.head.forward(h)

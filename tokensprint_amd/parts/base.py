@@ -1,0 +1,164 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A part is built from a `PartSpec` (its sizes and constants) and a `BuildContext`
+(kernels, dtype, device, shared position encodings).  It declares the checkpoint
+tensors it needs by full name, receives them once, and then only sees activations,
+the step's batch description and, for a mixer, the cache of the run it executes.
+No part knows which model it is in.
+
+Registries map a `kind` string to a class, one registry per role:
+`MIXERS`, `FEED_FORWARDS`, `NORMS`, `POSITIONS`, `BLOCKS`.  A test or a new
+architecture adds a part with `register(MIXERS, "my_kind")(MyClass)`.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable
+
+import torch
+
+
+# ------------------------------------------------------------------ declarations
+
+
+@dataclass(frozen=True)
+class TensorDecl:
+    """A checkpoint tensor a part needs.
+
+    role "matrix": used in a matrix product or as an embedding table; kept in the
+    run dtype unless the file stores it in 32-bit.  role "vector": a small per-
+    channel vector (norm weight); always held in float32, which is exact for
+    bfloat16 values.  role "table": an integer table, held as int32.
+    """
+
+    shape: tuple[int, ...]
+    role: str = "matrix"
+    optional: bool = False      # may be absent from the file (e.g. a tied head's copy)
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values per token, in pages.  window None = every earlier key."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class SlotStateNeed:
+    """A fixed-size per-request state tensor (shape without the slot axis)."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class BuildContext:
+    ops: Any                    # kernel provider (see tokensprint_amd.kernels)
+    dtype: torch.dtype          # activation dtype: bfloat16 or float32
+    device: torch.device
+    width: int
+    positions: dict[str, "PositionEncoding"] = field(default_factory=dict)
+
+
+# ------------------------------------------------------------------ part roles
+
+
+class Part:
+    def __init__(self, spec_params: dict, ctx: BuildContext) -> None:
+        self.params = dict(spec_params)
+        self.ctx = ctx
+        self.ops = ctx.ops
+
+    def tensors(self) -> dict[str, TensorDecl]:
+        """Checkpoint name -> declaration, for every tensor this part reads."""
+        return {}
+
+    def load(self, get: Callable[[str], torch.Tensor | None]) -> None:
+        """Take the declared tensors (`get(name)`, None if optional and absent)."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Normalised copy of x [T, width] in the activation dtype."""
+        raise NotImplementedError
+
+    def add_forward(self, resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+        """resid += delta (float32, in place), then the norm of the new resid."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Applied by a mixer to its queries and keys.
+
+    `rotary_tables()` returns (cos, sin) float32 [max_position, dim/2] for the
+    fused rotate-half kernel, or None; then the mixer calls `apply` instead.
+    """
+
+    def rotary_tables(self):
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor | None, positions: torch.Tensor) -> None:
+        """Encode positions into q [T, nq, hd] and k [T, nkv, hd] in place."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self) -> PagedKVNeed | SlotStateNeed | None:
+        return None
+
+    def forward(self, h: torch.Tensor, batch, cache, write_cache: bool) -> torch.Tensor:
+        """h [T, width] -> [T, width].  `cache` is this run's cache view (or None)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of one layer's parts around the residual stream.
+
+    The stream travels as (resid, delta): resid is float32 [T, width]; delta is
+    the last sub-layer's output not yet added (None at the very start), so the
+    add can be fused into the next norm.
+    """
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
+                 ffn_norm: Norm, ctx: BuildContext) -> None:
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+        self.ctx = ctx
+
+    def parts(self) -> list[Part]:
+        return [self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward]
+
+    def forward(self, resid, delta, batch, cache, write_cache: bool):
+        raise NotImplementedError
+
+
+# ------------------------------------------------------------------ registries
+
+MIXERS: dict[str, type] = {}
+FEED_FORWARDS: dict[str, type] = {}
+NORMS: dict[str, type] = {}
+POSITIONS: dict[str, type] = {}
+BLOCKS: dict[str, type] = {}
+
+
+def register(registry: dict[str, type], kind: str, *, replace: bool = False):
+    def deco(cls):
+        if kind in registry and not replace:
+            raise ValueError(f"part kind '{kind}' already registered")
+        registry[kind] = cls
+        return cls
+    return deco
+
+
+def build_part(registry: dict[str, type], spec, ctx: BuildContext):
+    if spec.kind not in registry:
+        raise ValueError(f"unknown part kind '{spec.kind}'; registered: {sorted(registry)}")
+    return registry[spec.kind](dict(spec.params), ctx)

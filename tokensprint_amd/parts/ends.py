@@ -1,0 +1,56 @@
+"""The two ends of a model: token embedding and the output head.
+
+Embedding: x[t] = E[ids[t]] (engine/model.py:65).  Head: tied, logits = x E^T over
+the embedding's own storage (engine/nn/layers.py:14-30); untied, x W^T without bias
+(HF lm_head has none; the reference's default-bias nn.Linear,
+engine/models/_builder.py:96, is not copied).  Logits leave in float32.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokensprint_amd.parts.base import Part, TensorDecl
+
+
+class Embedding(Part):
+    """params: weight (checkpoint name), vocab_size."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.name = params["weight"]
+        self.vocab = int(params["vocab_size"])
+        self.table = None
+
+    def tensors(self):
+        return {self.name: TensorDecl((self.vocab, self.ctx.width))}
+
+    def load(self, get):
+        self.table = get(self.name)
+
+    def forward(self, token_ids):
+        return self.ops.embed(self.table, token_ids)
+
+
+class Head(Part):
+    """params: weight (name), vocab_size, tied (bool: `weight` is the embedding's)."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.name = params["weight"]
+        self.vocab = int(params["vocab_size"])
+        self.tied = bool(params.get("tied", False))
+        self.ignored = params.get("ignored")      # a tied file's redundant copy
+        self.weight = None
+
+    def tensors(self):
+        t = {self.name: TensorDecl((self.vocab, self.ctx.width))}
+        if self.ignored:
+            t[self.ignored] = TensorDecl((self.vocab, self.ctx.width), optional=True)
+        return t
+
+    def load(self, get):
+        self.weight = get(self.name)
+
+    def forward(self, h):
+        return self.ops.linear(h, self.weight, torch.float32)

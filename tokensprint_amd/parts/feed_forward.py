@@ -1,0 +1,39 @@
+"""Dense SwiGLU feed-forward: down(silu(gate(h)) * up(h)), no bias
+(engine/nn/layers.py:61-66).  Gate and up run as one product over row-concatenated
+weights; the activation kernel reads both halves."""
+
+from __future__ import annotations
+
+import torch
+
+from tokensprint_amd.parts.base import FEED_FORWARDS, FeedForward, TensorDecl, register
+
+
+@register(FEED_FORWARDS, "swiglu")
+class SwiGLU(FeedForward):
+    """params: prefix, inner_dim."""
+
+    def __init__(self, params, ctx):
+        super().__init__(params, ctx)
+        self.prefix = params["prefix"]
+        self.inner = int(params["inner_dim"])
+        self.w_gate_up = self.w_down = None
+
+    def tensors(self):
+        H, I, pre = self.ctx.width, self.inner, self.prefix
+        return {pre + "gate_proj.weight": TensorDecl((I, H)),
+                pre + "up_proj.weight": TensorDecl((I, H)),
+                pre + "down_proj.weight": TensorDecl((H, I))}
+
+    def load(self, get):
+        pre = self.prefix
+        g, u = get(pre + "gate_proj.weight"), get(pre + "up_proj.weight")
+        if g.dtype != u.dtype:
+            raise ValueError(f"{pre}: gate and up weights are stored in different dtypes")
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = get(pre + "down_proj.weight")
+
+    def forward(self, h, batch):
+        gu = self.ops.linear(h, self.w_gate_up, self.ctx.dtype)
+        act = self.ops.silu_mul(gu)
+        return self.ops.linear(act, self.w_down, self.ctx.dtype)
