@@ -1,0 +1,138 @@
+"""Ways of cutting the same requests into steps; all must give the plain logits.
+
+Each drive feeds token ids through `ModelRunner.step` and collects, per request, the
+logits at every position it asked for.  The plain implementation runs each request
+whole, without a cache.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokensprint_amd.engine import StepEntry
+
+
+class Collector:
+    def __init__(self):
+        self.rows = {}     # request id -> {position: logits row}
+
+    def take(self, entries, logits):
+        r = 0
+        for e in entries:
+            for w in e.want:
+                self.rows.setdefault(e.cache.request_id, {})[e.start + w] = logits[r].cpu()
+                r += 1
+        assert r == logits.shape[0]
+
+    def stacked(self, rid):
+        got = self.rows[rid]
+        return torch.stack([got[p] for p in sorted(got)]), sorted(got)
+
+
+def drive_whole(runner, requests):
+    """Each request alone, the whole prompt in one step, logits everywhere."""
+    col = Collector()
+    for rid, tokens in requests.items():
+        rc = runner.manager.admit(rid)
+        runner.manager.extend(rc, len(tokens))
+        entries = [StepEntry(rc, tokens, 0, list(range(len(tokens))))]
+        col.take(entries, runner.step(entries))
+        runner.manager.free(rc)
+    runner.manager.check()
+    return col
+
+
+def drive_prefill_then_decode(runner, requests, tail=32):
+    """Most of the request in one step, then the last `tail` tokens one by one."""
+    col = Collector()
+    for rid, tokens in requests.items():
+        rc = runner.manager.admit(rid)
+        head = max(1, len(tokens) - tail)
+        runner.manager.extend(rc, head)
+        entries = [StepEntry(rc, tokens[:head], 0, list(range(head)))]
+        col.take(entries, runner.step(entries))
+        for p in range(head, len(tokens)):
+            runner.manager.extend(rc, p + 1)
+            entries = [StepEntry(rc, tokens[p:p + 1], p, [0])]
+            col.take(entries, runner.step(entries))
+        runner.manager.free(rc)
+    runner.manager.check()
+    return col
+
+
+def drive_portions(runner, requests, sizes=(7, 2, 13, 3, 2, 29, 5, 2, 64, 11)):
+    """Portions of changing size, down to two tokens, not aligned to pages."""
+    col = Collector()
+    for rid, tokens in requests.items():
+        rc = runner.manager.admit(rid)
+        pos, i = 0, 0
+        while pos < len(tokens):
+            n = min(sizes[i % len(sizes)], len(tokens) - pos)
+            i += 1
+            runner.manager.extend(rc, pos + n)
+            entries = [StepEntry(rc, tokens[pos:pos + n], pos, list(range(n)))]
+            col.take(entries, runner.step(entries))
+            pos += n
+        runner.manager.free(rc)
+    runner.manager.check()
+    return col
+
+
+def drive_mixed(runner, requests, max_live=4, seed=0, decode_tail=12):
+    """Up to `max_live` live requests: portions of some beside single decoded tokens of
+    others in one step, requests admitted as others end, so pages are used again."""
+    g = torch.Generator().manual_seed(seed)
+    col = Collector()
+    waiting = list(requests.items())
+    live = {}       # rid -> [rc, tokens, pos]
+    steps = 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, tokens = waiting[0]
+            # admit only if the whole request will fit beside what the others still need
+            rc = runner.manager.admit(rid)
+            live[rid] = [rc, tokens, 0]
+            waiting.pop(0)
+        entries, ended = [], []
+        for rid, state in live.items():
+            rc, tokens, pos = state
+            remaining = len(tokens) - pos
+            if remaining <= decode_tail:
+                n = 1
+            else:
+                n = int(torch.randint(2, 24, (1,), generator=g))
+                n = min(n, remaining - decode_tail)
+            # sometimes leave a request out of a step
+            if len(live) > 1 and float(torch.rand(1, generator=g)) < 0.15:
+                continue
+            if not runner.manager.can_extend(rc, pos + n):
+                continue
+            runner.manager.extend(rc, pos + n)
+            entries.append(StepEntry(rc, tokens[pos:pos + n], pos, list(range(n))))
+            state[2] = pos + n
+            if state[2] == len(tokens):
+                ended.append(rid)
+        if not entries:
+            steps += 1
+            assert steps < 10000, "mixed drive makes no progress: pool too small"
+            continue
+        col.take(entries, runner.step(entries))
+        for rid in ended:
+            runner.manager.free(live.pop(rid)[0])
+        runner.manager.check()
+    return col
+
+
+def compare(col, plain_logits, rtol, atol):
+    """Compare every collected request with the plain logits; on failure name the first
+    wrong position."""
+    for rid, ref in plain_logits.items():
+        got, positions = col.stacked(rid)
+        assert positions == list(range(ref.shape[0])), f"{rid}: positions {positions[:5]}..."
+        bad = ~torch.isclose(got, ref, rtol=rtol, atol=atol)
+        if bad.any():
+            p = int(bad.any(dim=1).nonzero()[0])
+            err = (got[p] - ref[p]).abs().max()
+            raise AssertionError(
+                f"request {rid}: first wrong position {p} of {ref.shape[0]}, "
+                f"max abs error there {err:.3e}, overall {(got - ref).abs().max():.3e}")

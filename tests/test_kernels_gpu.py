@@ -1,0 +1,225 @@
+"""Each HIP kernel alone against its plain torch reference (tests/kernel_refs.py), in
+float32 and bfloat16, at sizes other than the engine's tiny models: widths and
+vocabularies that are no power of two, head sizes in steps of 16, odd head groupings."""
+
+import pytest
+import torch
+
+from kernel_refs import TorchOps
+from scenarios import paged_scenario
+
+pytestmark = pytest.mark.gpu
+
+REF = TorchOps()
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops(gpu_device):
+    from tokensprint_amd.kernels import load_hip_ops
+    return load_hip_ops(gpu_device)
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1.6e-2)
+
+
+def rand(shape, dtype, device, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(device)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("vocab,width", [(389, 96), (1000, 1030)])
+def test_embed_and_gather(ops, gpu_device, dtype, vocab, width):
+    table = rand((vocab, width), dtype, gpu_device, 0)
+    ids = torch.randint(0, vocab, (77,), dtype=torch.int32, device=gpu_device)
+    out = ops.embed(table, ids)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out, REF.embed(table, ids), rtol=0, atol=0)
+    rows = torch.tensor([5, 0, 76, 5], dtype=torch.int32, device=gpu_device)
+    x = out.to(dtype)
+    torch.testing.assert_close(ops.gather_rows(x, rows), REF.gather_rows(x, rows), rtol=0, atol=0)
+
+
+# shapes (257,1024) and (4*73,1024), weights U(-1,1), eps 1e-6 are the reference's own
+# parity vectors (tests/test_kernel_parity.py:234-262 of the reference)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width", [(257, 1024), (292, 1024), (33, 96), (5, 5120), (7, 50)])
+def test_rmsnorm(ops, gpu_device, dtype, rows, width):
+    x = rand((rows, width), dtype, gpu_device, 1)
+    w = (torch.rand(width, generator=torch.Generator().manual_seed(2)) * 2 - 1).to(gpu_device)
+    out = ops.rmsnorm(x, w, 1e-6, dtype)
+    torch.testing.assert_close(out.float(), REF.rmsnorm(x, w, 1e-6, dtype).float(), **tol(dtype))
+    torch.testing.assert_close(
+        out.float(), torch.nn.functional.rms_norm(x.float(), (width,), w, 1e-6),
+        **(tol(dtype) if dtype == torch.float32 else dict(rtol=1e-2, atol=3.2e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_rmsnorm_updates_the_residual(ops, gpu_device, dtype):
+    rows, width = 19, 1030
+    resid = rand((rows, width), torch.float32, gpu_device, 3)
+    delta = rand((rows, width), dtype, gpu_device, 4)
+    w = 1 + 0.1 * rand((width,), torch.float32, gpu_device, 5)
+    ref_resid = resid.clone()
+    ref = REF.add_rmsnorm(ref_resid, delta, w, 1e-5, dtype)
+    out = ops.add_rmsnorm(resid, delta, w, 1e-5, dtype)
+    torch.testing.assert_close(resid, ref_resid, rtol=0, atol=0)
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, gpu_device, dtype):
+    gu = rand((37, 2 * 150), dtype, gpu_device, 6, scale=3.0)
+    torch.testing.assert_close(ops.silu_mul(gu).float(), REF.silu_mul(gu).float(), **tol(dtype))
+    g, u = gu[:, :150].float(), gu[:, 150:].float()
+    torch.testing.assert_close(ops.silu_mul(gu).float(), torch.nn.functional.silu(g) * u,
+                               **tol(dtype))
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("x_dtype,w_dtype", [(torch.float32, torch.float32),
+                                             (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 389, 96), (7, 130, 50), (64, 64, 64), (100, 301, 1030),
+                                   (300, 77, 17)])
+def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
+    x = rand((M, K), x_dtype, gpu_device, 7)
+    w = rand((N, K), w_dtype, gpu_device, 8, scale=0.1)
+    out = ops.linear(x, w, out_dtype)
+    ref = x.double() @ w.double().T
+    t = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.double(), ref, **t)
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):
+    x = rand((70, 200), torch.float32, gpu_device, 9)
+    w = rand((150, 200), torch.float32, gpu_device, 10)
+    full = ops.linear(x, w, torch.float32)
+    one = ops.linear(x[33:34].contiguous(), w, torch.float32)
+    assert torch.equal(full[33:34], one)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,page", [(4, 2, 16, 4), (8, 2, 32, 16), (6, 3, 48, 8),
+                                            (16, 8, 128, 16), (5, 5, 80, 3), (8, 1, 256, 64)])
+def test_qk_norm_rope_store(ops, gpu_device, dtype, nq, nkv, hd, page):
+    spans = [(0, 9), (13, 1), (5, 20), (31, 2)]
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=11)
+    T = batch.num_tokens
+    qkv = rand((T, (nq + 2 * nkv) * hd), dtype, gpu_device, 12)
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 13)
+    wk = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 14)
+    angles = torch.outer(torch.arange(64, dtype=torch.float32),
+                         1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    ref_cache = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                            cache.k_pages.clone(), cache.v_pages.clone())
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, q_weight=wq, k_weight=wk, eps=1e-5,
+              cos_sin=cos_sin)
+    q_ref = REF.qk_norm_rope_store(qkv, batch, table, ref_cache, **kw)
+    q = ops.qk_norm_rope_store(qkv, batch, table, cache, **kw)
+    torch.testing.assert_close(q.float(), q_ref.float(), **tol(dtype))
+    torch.testing.assert_close(cache.k_pages.float(), ref_cache.k_pages.float(), **tol(dtype))
+    torch.testing.assert_close(cache.v_pages.float(), ref_cache.v_pages.float(), rtol=0, atol=0)
+    # pieces alone: norm-only split, rotation in place, store
+    q2, k2, v2 = ops.qk_norm_split(qkv, num_heads=nq, num_kv_heads=nkv, head_dim=hd,
+                                   q_weight=wq, k_weight=wk, eps=1e-5)
+    q2r, k2r, v2r = REF.qk_norm_split(qkv, num_heads=nq, num_kv_heads=nkv, head_dim=hd,
+                                      q_weight=wq, k_weight=wk, eps=1e-5)
+    torch.testing.assert_close(q2.float(), q2r.float(), **tol(dtype))
+    torch.testing.assert_close(k2.float(), k2r.float(), **tol(dtype))
+    torch.testing.assert_close(v2.float(), v2r.float(), rtol=0, atol=0)
+    ops.rope_inplace(q2, batch.positions, *cos_sin)
+    REF.rope_inplace(q2r, batch.positions, *cos_sin)
+    torch.testing.assert_close(q2.float(), q2r.float(), **tol(dtype))
+    cache.k_pages.zero_(); ref_cache.k_pages.zero_()
+    ops.kv_store(k2, v2, batch, table, cache)
+    REF.kv_store(k2r, v2r, batch, table, ref_cache)
+    torch.testing.assert_close(cache.k_pages.float(), ref_cache.k_pages.float(), **tol(dtype))
+
+
+# the reference's rotary parity vector: 257 tokens, 16/8 heads of 128, positions below
+# 4096, theta 1e6 (tests/test_kernel_parity.py:71-109 of the reference)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_reference_shape(ops, gpu_device, dtype):
+    hd, max_pos = 128, 4096
+    angles = torch.outer(torch.arange(max_pos, dtype=torch.float32),
+                         1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos, sin = angles.cos().to(gpu_device), angles.sin().to(gpu_device)
+    pos = torch.randint(0, max_pos, (257,), dtype=torch.int32, device=gpu_device)
+    for heads in (16, 8):
+        x = rand((257, heads, hd), dtype, gpu_device, 15 + heads)
+        ref = x.clone()
+        ops.rope_inplace(x, pos, cos, sin)
+        REF.rope_inplace(ref, pos, cos, sin)
+        t = tol(dtype) if dtype == torch.float32 else dict(rtol=1e-2, atol=2e-2)
+        torch.testing.assert_close(x.float(), ref.float(), **t)
+
+
+ATTN_SHAPES = [(4, 2, 16, 4), (8, 2, 32, 16), (6, 3, 48, 8), (16, 8, 128, 16), (5, 5, 80, 3),
+               (8, 1, 64, 64), (4, 4, 256, 16), (14, 2, 112, 32)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 7, 40])
+@pytest.mark.parametrize("nq,nkv,hd,page", ATTN_SHAPES)
+def test_paged_attention(ops, gpu_device, dtype, nq, nkv, hd, page, window):
+    spans = [(0, 9), (70, 1), (5, 33), (130, 2), (0, 1), (63, 1), (64, 1), (65, 70)]
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=21)
+    q = rand((batch.num_tokens, nq, hd), dtype, gpu_device, 22)
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
+    out = ops.paged_attention(q, batch, table, cache, **kw)
+    ref = REF.paged_attention(q, batch, table, cache, **kw)
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
+    """One key among hundreds, at a page's edge, is made to dominate: the output must be
+    its value row.  A kernel that skips a tile, a page or the last key of a page fails."""
+    nq, nkv, hd, page = 4, 2, 64, 16
+    for far in (0, 15, 16, 255, 256, 511, 700):
+        batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                                spans=[(700, 1)], seed=23)
+        q = rand((1, nq, hd), dtype, gpu_device, 24)
+        phys = int(table[0, far // page])
+        for kvh in range(nkv):
+            # key = 4 * q of the first head of the group: score is far above the others
+            cache.k_pages[phys, kvh, far % page] = (4.0 * q[0, kvh * 2]).to(dtype)
+        out = ops.paged_attention(q, batch, table, cache, num_heads=nq, num_kv_heads=nkv,
+                                  head_dim=hd, scale=1.0, window=None)
+        for kvh in range(nkv):
+            torch.testing.assert_close(out[0, kvh * 2].float(),
+                                       cache.v_pages[phys, kvh, far % page].float(),
+                                       rtol=2e-2, atol=2e-2)
+
+
+def test_argmax_and_ties(ops, gpu_device):
+    logits = rand((9, 151936), torch.float32, gpu_device, 30)
+    assert torch.equal(ops.argmax(logits).long(), logits.argmax(-1))
+    logits = torch.zeros(3, 389, device=gpu_device)
+    logits[0, 17] = logits[0, 300] = 2.0
+    logits[1, 388] = 1.0
+    assert ops.argmax(logits).tolist() == [17, 388, 0]
+
+
+def test_sample_is_keyed_and_follows_the_distribution(ops, gpu_device):
+    vocab = 11
+    logits = torch.linspace(-2, 2, vocab, device=gpu_device).repeat(4000, 1).contiguous()
+    temps = torch.full((4000,), 0.7, device=gpu_device)
+    keys = torch.arange(4000, dtype=torch.int64, device=gpu_device) * 7919 + 5
+    a = ops.sample(logits, temps, keys)
+    # same key, other batch: same token
+    b = ops.sample(logits[100:200].contiguous(), temps[100:200].contiguous(),
+                   keys[100:200].contiguous())
+    assert torch.equal(a[100:200], b)
+    freq = torch.bincount(a.long(), minlength=vocab).float() / 4000
+    probs = torch.softmax(logits[0] / 0.7, -1)
+    assert (freq - probs).abs().max() < 0.03
+    # temperature 0 rows are greedy
+    temps[:10] = 0.0
+    assert (ops.sample(logits, temps, keys)[:10] == vocab - 1).all()

@@ -1,0 +1,110 @@
+// Paged causal attention for any head size up to 256, any page size, any head grouping,
+// float32 or bfloat16 storage, float32 arithmetic throughout: the attention of the
+// float32 path and of shapes the matrix-core kernels do not take.
+//
+// One wavefront per (query token, query head).  Keys are walked in tiles of 64 starting
+// at the first visible key, so the partition, and with it the rounding, depends only on
+// the token's position and the window, never on how the step was cut or batched.
+#include "attention.h"
+
+constexpr int kMaxHeadDim = 256;
+constexpr int kWavesPerBlock = 4;
+
+template <typename T, typename TC>
+__global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kernel(AttentionArgs a) {
+  __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
+  __shared__ float p_s[kWavesPerBlock][kWave];
+  __shared__ int64_t row_s[kWavesPerBlock][kWave];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t item = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  if (item >= (int64_t)a.num_tokens * a.nq) return;   // whole wave leaves together
+  const int t = (int)(item / a.nq), h = (int)(item % a.nq);
+  const int kvh = h / (a.nq / a.nkv);
+  const int hd = a.hd, P = a.page_size;
+  const int pos = a.positions[t];
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int* table = a.table + (int64_t)a.entry_of_token[t] * a.table_width;
+  const T* q = (const T*)a.q + item * hd;
+  const TC* kp = (const TC*)a.k_pages;
+  const TC* vp = (const TC*)a.v_pages;
+
+  for (int d = lane; d < hd; d += kWave) q_s[wave][d] = to_f32(q[d]);
+  // a wavefront runs in lockstep and only reads its own rows of LDS: no barrier needed,
+  // but the compiler must not reorder the LDS traffic
+  __builtin_amdgcn_wave_barrier();
+
+  float m = -INFINITY, l = 0.f;
+  float acc[kMaxHeadDim / kWave] = {};
+  for (int j0 = lo; j0 <= pos; j0 += kWave) {
+    const int j = j0 + lane;
+    const bool valid = j <= pos;
+    float s = -INFINITY;
+    int64_t row = -1;
+    if (valid) {
+      const int page = table[j / P];
+      if (page >= 0) {
+        row = (((int64_t)page * a.nkv + kvh) * P + j % P) * hd;
+        const TC* kr = kp + row;
+        float dot = 0.f;
+        for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
+        s = dot * a.scale;
+      }
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    // m_new stays -inf only while no key has been seen (pages given back): keep zeros
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);   // exp(-inf) = 0 at first
+    const float p = (row >= 0 && m_new != -INFINITY) ? expf(s - m_new) : 0.f;
+    l = l * corr + wave_sum(p);
+    p_s[wave][lane] = p;
+    row_s[wave][lane] = row;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < kMaxHeadDim / kWave; ++r) acc[r] *= corr;
+    const int n = min(kWave, pos - j0 + 1);
+    for (int jj = 0; jj < n; ++jj) {
+      const int64_t vrow = row_s[wave][jj];
+      if (vrow < 0) continue;
+      const float pj = p_s[wave][jj];
+#pragma unroll
+      for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+        const int d = lane + r * kWave;
+        if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vrow + d]), acc[r]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    m = m_new;
+  }
+  T* o = (T*)a.out + item * hd;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+    const int d = lane + r * kWave;
+    if (d < hd) o[d] = from_f32<T>(acc[r] * inv);
+  }
+}
+
+int ts_check_attention_args(const AttentionArgs& a, const char* who) {
+  if (a.hd <= 0 || a.hd > kMaxHeadDim) TS_FAIL("%s: head_dim=%d not in 1..%d", who, a.hd, kMaxHeadDim);
+  if (a.nq <= 0 || a.nkv <= 0 || a.nq % a.nkv)
+    TS_FAIL("%s: %d query heads cannot share %d key/value heads", who, a.nq, a.nkv);
+  if (a.page_size <= 0 || a.table_width <= 0 || a.num_pages <= 0)
+    TS_FAIL("%s: page_size=%d table_width=%d num_pages=%d", who, a.page_size, a.table_width,
+            a.num_pages);
+  if (a.window < 0) TS_FAIL("%s: window=%d", who, a.window);
+  return 0;
+}
+
+extern "C" int ts_attention_generic(const AttentionArgs* args, int act_type, int cache_type,
+                                    hipStream_t stream) {
+  AttentionArgs a = *args;
+  if (a.num_tokens <= 0) return 0;
+  if (ts_check_attention_args(a, "attention_generic")) return -1;
+  const int64_t items = (int64_t)a.num_tokens * a.nq;
+  const int64_t blocks = (items + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (blocks > 2147483647LL) TS_FAIL("attention_generic: too many tokens");
+  TS_DISPATCH_TYPE(act_type, T, TS_DISPATCH_TYPE(cache_type, TC,
+      hipLaunchKernelGGL((attention_generic_kernel<T, TC>), dim3((unsigned)blocks),
+                         dim3(kWavesPerBlock * kWave), 0, stream, a)));
+  TS_CHECK_LAUNCH("attention_generic");
+  return 0;
+}

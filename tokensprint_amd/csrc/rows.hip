@@ -1,0 +1,123 @@
+// Row-wise kernels: embedding gather, row gather, RMSNorm (with and without the fused
+// residual add), SiLU-multiply.  One workgroup per row; sums in float32.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int width) {
+  const int64_t t = blockIdx.x;
+  const TW* row = table + (int64_t)ids[t] * width;
+  float* o = out + t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]);
+}
+
+extern "C" int ts_embed(const void* table, int table_type, int vocab, const int* ids,
+                        float* out, int num_tokens, int width, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (width <= 0 || vocab <= 0) TS_FAIL("embed: bad sizes width=%d vocab=%d", width, vocab);
+  TS_DISPATCH_TYPE(table_type, TW,
+                   hipLaunchKernelGGL(embed_kernel<TW>, dim3(num_tokens), dim3(256), 0, stream,
+                                      (const TW*)table, ids, out, width));
+  TS_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- row gather
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ rows,
+                                   T* __restrict__ out, int width) {
+  const int64_t r = blockIdx.x;
+  const T* src = x + (int64_t)rows[r] * width;
+  T* dst = out + r * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int ts_gather_rows(const void* x, int type, const int* rows, void* out,
+                              int num_rows, int width, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  TS_DISPATCH_TYPE(type, T,
+                   hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(num_rows), dim3(256), 0,
+                                      stream, (const T*)x, rows, (T*)out, width));
+  TS_CHECK_LAUNCH("gather_rows");
+  return 0;
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// out = x * rsqrt(mean(x^2) + eps) * w.  With `delta`, first resid += delta (float32,
+// written back) and the norm is taken of the sum.
+template <typename TX, typename TD, typename TO, bool ADD>
+__global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
+                               const float* __restrict__ w, TO* __restrict__ out, int width,
+                               float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  TX* xr = x + row * width;
+  const TD* dr = ADD ? delta + row * width : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = to_f32(xr[i]);
+    if (ADD) {
+      v += to_f32(dr[i]);
+      xr[i] = from_f32<TX>(v);
+    }
+    ss += v * v;
+  }
+  const float rstd = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  TO* o = out + row * width;
+  // each thread re-reads what it wrote itself, so no barrier is needed for x
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    o[i] = from_f32<TO>(to_f32(xr[i]) * rstd * w[i]);
+}
+
+extern "C" int ts_rmsnorm(const void* x, int x_type, const float* w, void* out, int out_type,
+                          int rows, int width, float eps, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0) TS_FAIL("rmsnorm: width=%d", width);
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  TS_DISPATCH_TYPE(x_type, TX, TS_DISPATCH_TYPE(out_type, TO,
+      hipLaunchKernelGGL((rmsnorm_kernel<TX, float, TO, false>), dim3(rows), dim3(threads), 0,
+                         stream, (TX*)x, (const float*)nullptr, w, (TO*)out, width, eps)));
+  TS_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+extern "C" int ts_add_rmsnorm(float* resid, const void* delta, int delta_type, const float* w,
+                              void* out, int out_type, int rows, int width, float eps,
+                              hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0) TS_FAIL("add_rmsnorm: width=%d", width);
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  TS_DISPATCH_TYPE(delta_type, TD, TS_DISPATCH_TYPE(out_type, TO,
+      hipLaunchKernelGGL((rmsnorm_kernel<float, TD, TO, true>), dim3(rows), dim3(threads), 0,
+                         stream, resid, (const TD*)delta, w, (TO*)out, width, eps)));
+  TS_CHECK_LAUNCH("add_rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------- SiLU(gate) * up
+// gate_up is [rows, 2*inner]: gate in the first half of a row, up in the second.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t total,
+                                int inner) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / inner;
+    const int c = (int)(i - r * inner);
+    const float g = to_f32(gu[r * 2 * inner + c]);
+    const float u = to_f32(gu[r * 2 * inner + inner + c]);
+    out[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ts_silu_mul(const void* gate_up, void* out, int type, int rows, int inner,
+                           hipStream_t stream) {
+  if (rows <= 0) return 0;
+  const int64_t total = (int64_t)rows * inner;
+  const int blocks = (int)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256);
+  TS_DISPATCH_TYPE(type, T,
+                   hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, stream,
+                                      (const T*)gate_up, (T*)out, total, inner));
+  TS_CHECK_LAUNCH("silu_mul");
+  return 0;
+}

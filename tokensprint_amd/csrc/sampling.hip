@@ -1,0 +1,79 @@
+// Sampling over float32 logits [R, V]: argmax, and temperature sampling by
+// argmax(logit/T - log E) with E ~ Exp(1), which picks token i with probability
+// softmax(logits/T)[i].  The noise of (row, vocabulary index) comes from a counter hash
+// keyed per row, so a token does not depend on what else is in the batch.
+#include "common.h"
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+  return z ^ (z >> 31);
+}
+
+// uniform in (0, 1) from 24 bits
+__device__ __forceinline__ float uniform01(uint64_t key, uint32_t index) {
+  const uint64_t z = mix64(key + 0x9E3779B97F4A7C15ULL * (uint64_t)(index + 1));
+  return ((float)(uint32_t)(z >> 40) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+struct Best { float v; int i; };
+__device__ __forceinline__ Best better(Best a, Best b) {
+  // larger value wins; equal values: lower index
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+
+template <bool NOISE>
+__global__ __launch_bounds__(256) void pick_kernel(const float* __restrict__ logits,
+                                                   const float* __restrict__ temperature,
+                                                   const uint64_t* __restrict__ keys,
+                                                   int* __restrict__ out, int vocab) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int r = blockIdx.x;
+  const float* row = logits + (int64_t)r * vocab;
+  const float temp = NOISE ? temperature[r] : 1.f;
+  const bool noisy = NOISE && temp > 1e-10f;
+  const float inv_t = noisy ? 1.f / temp : 1.f;
+  const uint64_t key = NOISE ? keys[r] : 0;
+  Best best{-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    float s = row[i];
+    if (noisy) {
+      const float e = fmaxf(-logf(uniform01(key, (uint32_t)i)), 1e-10f);
+      s = s * inv_t - logf(e);
+    }
+    best = better(best, Best{s, i});
+  }
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1)
+    best = better(best, Best{__shfl_xor(best.v, o, kWave), __shfl_xor(best.i, o, kWave)});
+  const int wave = threadIdx.x / kWave;
+  if (threadIdx.x % kWave == 0) { sv[wave] = best.v; si[wave] = best.i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best b{sv[0], si[0]};
+    for (int w = 1; w < 4; ++w) b = better(b, Best{sv[w], si[w]});
+    out[r] = b.i;
+  }
+}
+
+extern "C" int ts_argmax(const float* logits, int* out, int rows, int vocab,
+                         hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) TS_FAIL("argmax: vocab=%d", vocab);
+  hipLaunchKernelGGL(pick_kernel<false>, dim3(rows), dim3(256), 0, stream, logits,
+                     (const float*)nullptr, (const uint64_t*)nullptr, out, vocab);
+  TS_CHECK_LAUNCH("argmax");
+  return 0;
+}
+
+// temperature[r] <= 1e-10 means greedy for that row.
+extern "C" int ts_sample(const float* logits, const float* temperature, const uint64_t* keys,
+                         int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) TS_FAIL("sample: vocab=%d", vocab);
+  hipLaunchKernelGGL(pick_kernel<true>, dim3(rows), dim3(256), 0, stream, logits, temperature,
+                     keys, out, vocab);
+  TS_CHECK_LAUNCH("sample");
+  return 0;
+}

@@ -33,9 +33,11 @@ def build_model(raw_config: dict, dtype, device, ops=None):
     """(typed config, Model without weights) for a raw config.json dict."""
     dtype = parse_dtype(dtype)
     device = torch.device(device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", 0)
     if ops is None:
-        from tokensprint_amd.kernels import hip_ops
-        ops = hip_ops(device)
+        from tokensprint_amd.kernels import load_hip_ops
+        ops = load_hip_ops(device)
     arch = get_architecture(architecture_of(raw_config))
     config = arch.parse_config(raw_config)
     spec = arch.build_spec(config)

@@ -1,0 +1,140 @@
+"""Python entry point: LLMEngine(model, config, tokenizer).generate(prompts, params).
+
+Surface of the reference's engine/generation/llm_engine.py:18-114: `add_request`,
+`step` (schedule -> run -> postprocess), `generate` (enqueue all, loop until the
+scheduler is empty, completions in request order), `is_finished`.  The tokenizer is
+optional: prompts given as token-id lists need none.
+"""
+
+from __future__ import annotations
+
+import logging
+import time
+
+import torch
+
+from tokensprint_amd.config.engine_config import Config, SamplingParams
+from tokensprint_amd.engine.batch import StepEntry
+from tokensprint_amd.engine.request import Request
+from tokensprint_amd.engine.runner import ModelRunner
+from tokensprint_amd.engine.scheduler import Scheduler
+from tokensprint_amd.models.model import Model
+from tokensprint_amd.sampling.sampler import Sampler
+
+log = logging.getLogger(__name__)
+
+
+class LLMEngine:
+    def __init__(self, model: Model, config: Config, tokenizer=None) -> None:
+        self.model, self.config, self.tokenizer = model, config, tokenizer
+        if model.ctx.dtype != config.dtype:
+            raise ValueError(f"model runs in {model.ctx.dtype}, config asks for {config.dtype}")
+        page = config.kvcache_block_size
+        num_pages = config.num_kvcache_blocks
+        if num_pages < 0:
+            num_pages = self._pages_from_free_memory(model, config)
+            config.num_kvcache_blocks = num_pages
+        self.runner = ModelRunner(model, page_size=page, num_pages=num_pages,
+                                  num_slots=config.max_num_seqs)
+        self.scheduler = Scheduler(
+            self.runner.manager, max_num_batched_tokens=config.max_num_batched_tokens,
+            max_num_seqs=config.max_num_seqs, max_model_len=config.max_model_len,
+            eos=config.eos, chunked_prefill=config.chunked_prefill)
+        self.sampler = Sampler(model.ctx.ops, model.ctx.device, config.seed)
+        self._next_ordinal = 0
+        self.requests: dict[int, Request] = {}
+
+    @staticmethod
+    def _pages_from_free_memory(model: Model, config: Config) -> int:
+        """free * utilization minus room for one step's activations, in pages
+        (engine/generation/model_runner.py:392-411)."""
+        device = model.ctx.device
+        if device.type != "cuda":
+            raise ValueError("num_kvcache_blocks must be given when there is no GPU to size from")
+        free, _ = torch.cuda.mem_get_info(device)
+        spec = model.spec
+        widest = max(spec.width * 8, spec.vocab_size // 8)
+        act = config.max_num_batched_tokens * widest * 4 * 4
+        logits = min(config.max_num_seqs, config.max_num_batched_tokens) * spec.vocab_size * 4 * 2
+        available = free * config.gpu_memory_utilization - act - logits
+        pages = ModelRunner.pages_that_fit(model, config.kvcache_block_size, int(available),
+                                           config.dtype)
+        # no request can use more than max_model_len tokens
+        cap = config.max_num_seqs * (-(-config.max_model_len // config.kvcache_block_size) + 1)
+        pages = min(pages, cap)
+        if pages < 1:
+            raise RuntimeError("Insufficient GPU memory for the key/value cache: "
+                               f"available={int(available)} bytes")
+        return pages
+
+    # ------------------------------------------------------------ requests
+    def _tokenize_prompt(self, prompt: str) -> list[int]:
+        if self.tokenizer is None:
+            raise ValueError("a text prompt needs a tokenizer; pass token ids instead")
+        token_ids = self.tokenizer.encode(prompt, add_special_tokens=True)
+        if not isinstance(token_ids, list):
+            raise TypeError("Expected tokenizer.encode(...) to return list[int].")
+        return token_ids
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    def add_request(self, prompt: str | list[int], sampling_params: SamplingParams) -> int:
+        if isinstance(prompt, str):
+            prompt = self._tokenize_prompt(prompt)
+        vocab = self.model.spec.vocab_size
+        if any(not 0 <= t < vocab for t in prompt):
+            raise ValueError(f"prompt holds a token id outside [0, {vocab})")
+        req = Request(self._next_ordinal, prompt, sampling_params)
+        self.scheduler.add_request(req)
+        self._next_ordinal += 1
+        self.requests[req.ordinal] = req
+        return req.ordinal
+
+    # ------------------------------------------------------------ one step
+    def step(self):
+        reqs = self.scheduler.schedule()
+        entries, sampled_index = [], []
+        for i, req in enumerate(reqs):
+            lo, hi = req.num_cached_tokens, req.num_cached_tokens + req.num_new_tokens
+            last = hi == len(req)
+            if last:
+                sampled_index.append(i)
+            entries.append(StepEntry(req.cache, req.token_ids[lo:hi], lo,
+                                     [req.num_new_tokens - 1] if last else []))
+        logits = self.runner.step(entries)
+        token_ids = self.sampler(logits, [reqs[i] for i in sampled_index])
+        self.scheduler.postprocess(reqs, token_ids, sampled_index)
+        outputs = [(r.ordinal, r.completion_token_ids) for r in reqs if r.is_finished]
+        num_total_tokens = sum(len(r) for r in reqs if r.is_finished)
+        for r in reqs:
+            if r.is_finished:
+                self.requests.pop(r.ordinal, None)
+        return outputs, num_total_tokens
+
+    def generate(self, prompts, sampling_params, use_tqdm: bool = True) -> list[list[int]]:
+        if not isinstance(sampling_params, list):
+            sampling_params = [sampling_params] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("sampling_params length must match prompts length, "
+                             f"got {len(sampling_params)} and {len(prompts)}.")
+        pbar = None
+        if use_tqdm:
+            from tqdm.auto import tqdm
+            pbar = tqdm(total=len(prompts), desc="Generating", dynamic_ncols=True)
+        ordinals = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        outputs: dict[int, list[int]] = {}
+        total, t0 = 0, time.perf_counter()
+        while not self.is_finished():
+            finished, n = self.step()
+            total += n
+            for ordinal, token_ids in finished:
+                outputs[ordinal] = token_ids
+                if pbar is not None:
+                    pbar.update(1)
+            if pbar is not None:
+                rate = total / max(time.perf_counter() - t0, 1e-9)
+                pbar.set_postfix({"total_throughput": f"{int(rate)}tok/s"})
+        if pbar is not None:
+            pbar.close()
+        return [outputs[o] for o in ordinals]

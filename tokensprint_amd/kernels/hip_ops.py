@@ -1,0 +1,312 @@
+"""The HIP kernels as Python operations: argument checks on the host, then one C call.
+
+Every method checks shapes, dtypes, devices and contiguity before a pointer reaches a
+kernel, because a kernel handed a wrong shape would read or write out of bounds.  There
+is no other implementation behind these methods: without a GPU or without the built
+library, construction raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
+
+import torch
+
+from tokensprint_amd.kernels.build import build, find_library
+
+ABI_VERSION = 1
+_TYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+class QkPrepareArgs(Structure):
+    _fields_ = [
+        ("qkv", c_void_p), ("q_out", c_void_p), ("k_dst", c_void_p), ("v_dst", c_void_p),
+        ("q_weight", c_void_p), ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p),
+        ("positions", c_void_p), ("entry_of_token", c_void_p), ("table", c_void_p),
+        ("table_width", c_int), ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int),
+        ("hd", c_int), ("page_size", c_int), ("max_pos", c_int), ("paged", c_int),
+        ("store_kv", c_int), ("eps", c_float),
+    ]
+
+
+class AttentionArgs(Structure):
+    _fields_ = [
+        ("q", c_void_p), ("out", c_void_p), ("k_pages", c_void_p), ("v_pages", c_void_p),
+        ("positions", c_void_p), ("entry_of_token", c_void_p), ("q_start", c_void_p),
+        ("ctx_len", c_void_p), ("table", c_void_p),
+        ("table_width", c_int), ("num_tokens", c_int), ("num_entries", c_int), ("nq", c_int),
+        ("nkv", c_int), ("hd", c_int), ("page_size", c_int), ("num_pages", c_int),
+        ("window", c_int), ("scale", c_float),
+    ]
+
+
+def _load_library() -> ctypes.CDLL:
+    path = find_library()
+    if path is None:
+        path = build()
+    lib = ctypes.CDLL(str(path))
+    lib.ts_last_error.restype = ctypes.c_char_p
+    if lib.ts_abi_version() != ABI_VERSION:
+        raise KernelError(f"{path} has interface version {lib.ts_abi_version()}, "
+                          f"this package needs {ABI_VERSION}")
+    return lib
+
+
+def _ptr(t: torch.Tensor | None):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+class HipOps:
+    name = "hip-gfx950"
+
+    def __init__(self, device) -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError(
+                "the HIP kernels need an AMD GPU (device 'cuda:N'); there is no CPU path")
+        self.lib = _load_library()
+
+    # ------------------------------------------------------------ helpers
+    def _stream(self):
+        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _call(self, fn, *args):
+        if fn(*args) != 0:
+            raise KernelError(self.lib.ts_last_error().decode())
+
+    def _check(self, name, t, dtype=None, shape=None, ndim=None):
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{name}: expected a tensor, got {type(t)}")
+        if t.device != self.device:
+            raise ValueError(f"{name}: on {t.device}, kernels run on {self.device}")
+        if not t.is_contiguous():
+            raise ValueError(f"{name}: must be contiguous, strides {t.stride()}")
+        if dtype is not None:
+            dtypes = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+            if t.dtype not in dtypes:
+                raise TypeError(f"{name}: dtype {t.dtype}, expected one of {dtypes}")
+        if ndim is not None and t.dim() != ndim:
+            raise ValueError(f"{name}: {t.dim()} dimensions, expected {ndim}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    _FLOATS = (torch.float32, torch.bfloat16)
+
+    # ------------------------------------------------------------ rows
+    def embed(self, table, token_ids):
+        self._check("embedding table", table, self._FLOATS, ndim=2)
+        self._check("token ids", token_ids, torch.int32, ndim=1)
+        T, (V, H) = token_ids.shape[0], table.shape
+        out = torch.empty(T, H, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_embed, _ptr(table), _TYPE_CODE[table.dtype], V, _ptr(token_ids),
+                   _ptr(out), T, H, self._stream())
+        return out
+
+    def gather_rows(self, x, rows):
+        self._check("x", x, self._FLOATS, ndim=2)
+        self._check("rows", rows, torch.int32, ndim=1)
+        out = torch.empty(rows.shape[0], x.shape[1], dtype=x.dtype, device=self.device)
+        self._call(self.lib.ts_gather_rows, _ptr(x), _TYPE_CODE[x.dtype], _ptr(rows), _ptr(out),
+                   rows.shape[0], x.shape[1], self._stream())
+        return out
+
+    def rmsnorm(self, x, weight, eps, out_dtype):
+        self._check("x", x, self._FLOATS, ndim=2)
+        self._check("norm weight", weight, torch.float32, shape=(x.shape[1],))
+        out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_rmsnorm, _ptr(x), _TYPE_CODE[x.dtype], _ptr(weight), _ptr(out),
+                   _TYPE_CODE[out_dtype], x.shape[0], x.shape[1], c_float(eps), self._stream())
+        return out
+
+    def add_rmsnorm(self, resid, delta, weight, eps, out_dtype):
+        self._check("resid", resid, torch.float32, ndim=2)
+        self._check("delta", delta, self._FLOATS, shape=resid.shape)
+        self._check("norm weight", weight, torch.float32, shape=(resid.shape[1],))
+        out = torch.empty(resid.shape, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_add_rmsnorm, _ptr(resid), _ptr(delta), _TYPE_CODE[delta.dtype],
+                   _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], resid.shape[0],
+                   resid.shape[1], c_float(eps), self._stream())
+        return out
+
+    def silu_mul(self, gate_up):
+        self._check("gate_up", gate_up, self._FLOATS, ndim=2)
+        rows, two_inner = gate_up.shape
+        if two_inner % 2:
+            raise ValueError("gate_up needs an even row width (gate half, up half)")
+        out = torch.empty(rows, two_inner // 2, dtype=gate_up.dtype, device=self.device)
+        self._call(self.lib.ts_silu_mul, _ptr(gate_up), _ptr(out), _TYPE_CODE[gate_up.dtype],
+                   rows, two_inner // 2, self._stream())
+        return out
+
+    # ------------------------------------------------------------ matrix product
+    def linear(self, x, weight, out_dtype):
+        """x [M, K] times weight [N, K] transposed -> [M, N] in out_dtype."""
+        self._check("x", x, self._FLOATS, ndim=2)
+        self._check("weight", weight, self._FLOATS, ndim=2)
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.shape[1] != K:
+            raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
+        out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_gemm_fma, _ptr(x), _TYPE_CODE[x.dtype], _ptr(weight),
+                   _TYPE_CODE[weight.dtype], _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                   self._stream())
+        return out
+
+    # ------------------------------------------------------------ q/k preparation
+    def _qk_args(self, qkv, batch, *, num_heads, kv_in_row, head_dim, q_weight, k_weight, eps,
+                 cos_sin):
+        T = qkv.shape[0]
+        self._check("qkv", qkv, self._FLOATS, shape=(T, (num_heads + 2 * kv_in_row) * head_dim))
+        if head_dim % 2:
+            raise ValueError(f"head_dim={head_dim} must be even")
+        a = QkPrepareArgs()
+        a.qkv = qkv.data_ptr()
+        a.num_tokens, a.nq, a.nkv, a.hd = T, num_heads, kv_in_row, head_dim
+        a.eps = eps
+        if q_weight is not None:
+            a.q_weight = self._check("q norm weight", q_weight, torch.float32,
+                                     shape=(head_dim,)).data_ptr()
+        if k_weight is not None:
+            a.k_weight = self._check("k norm weight", k_weight, torch.float32,
+                                     shape=(head_dim,)).data_ptr()
+        if cos_sin is not None:
+            cos, sin = cos_sin
+            self._check("cos", cos, torch.float32, ndim=2)
+            self._check("sin", sin, torch.float32, shape=cos.shape)
+            if cos.shape[1] != head_dim // 2:
+                raise ValueError(f"rotary table has {cos.shape[1]} columns, "
+                                 f"head_dim/2 is {head_dim // 2}")
+            if batch.max_ctx_len > cos.shape[0]:
+                raise ValueError(f"position {batch.max_ctx_len - 1} is beyond the rotary "
+                                 f"table's {cos.shape[0]} rows")
+            a.cos, a.sin, a.max_pos = cos.data_ptr(), sin.data_ptr(), cos.shape[0]
+        self._check("positions", batch.positions, torch.int32, shape=(T,))
+        self._check("entry_of_token", batch.entry_of_token, torch.int32, shape=(T,))
+        a.positions = batch.positions.data_ptr()
+        a.entry_of_token = batch.entry_of_token.data_ptr()
+        return a
+
+    def _check_cache(self, cache, table, batch, nkv, head_dim):
+        P = cache.page_size
+        self._check("k_pages", cache.k_pages, self._FLOATS,
+                    shape=(cache.num_pages, nkv, P, head_dim))
+        self._check("v_pages", cache.v_pages, cache.k_pages.dtype, shape=cache.k_pages.shape)
+        self._check("block table", table, torch.int32, ndim=2)
+        if table.shape[0] != batch.num_entries:
+            raise ValueError("block table rows differ from the batch's entries")
+        if table.shape[1] * P < batch.max_ctx_len:
+            raise ValueError(
+                f"block table of width {table.shape[1]} (page size {P}) cannot cover "
+                f"{batch.max_ctx_len} positions")
+
+    def qk_norm_rope_store(self, qkv, batch, table, cache, *, num_heads, num_kv_heads,
+                           head_dim, q_weight, k_weight, eps, cos_sin):
+        a = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=num_kv_heads,
+                          head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
+                          cos_sin=cos_sin)
+        q = torch.empty(qkv.shape[0], num_heads, head_dim, dtype=qkv.dtype, device=self.device)
+        a.q_out = q.data_ptr()
+        cache_type = _TYPE_CODE[qkv.dtype]
+        if cache is not None and num_kv_heads:
+            self._check_cache(cache, table, batch, num_kv_heads, head_dim)
+            a.k_dst, a.v_dst = cache.k_pages.data_ptr(), cache.v_pages.data_ptr()
+            a.table, a.table_width = table.data_ptr(), table.shape[1]
+            a.page_size, a.paged, a.store_kv = cache.page_size, 1, 1
+            cache_type = _TYPE_CODE[cache.k_pages.dtype]
+        self._call(self.lib.ts_qk_prepare, byref(a), _TYPE_CODE[qkv.dtype], cache_type,
+                   self._stream())
+        return q
+
+    def qk_norm_split(self, qkv, *, num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps):
+        T = qkv.shape[0]
+
+        class _B:   # positions are not used without a rotation or a paged store
+            positions = torch.zeros(T, dtype=torch.int32, device=self.device)
+            entry_of_token = positions
+            max_ctx_len = 0
+        a = self._qk_args(qkv, _B, num_heads=num_heads, kv_in_row=num_kv_heads,
+                          head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
+                          cos_sin=None)
+        q = torch.empty(T, num_heads, head_dim, dtype=qkv.dtype, device=self.device)
+        a.q_out = q.data_ptr()
+        k = v = None
+        if num_kv_heads:
+            k = torch.empty(T, num_kv_heads, head_dim, dtype=qkv.dtype, device=self.device)
+            v = torch.empty_like(k)
+            a.k_dst, a.v_dst, a.paged, a.store_kv = k.data_ptr(), v.data_ptr(), 0, 1
+        self._call(self.lib.ts_qk_prepare, byref(a), _TYPE_CODE[qkv.dtype],
+                   _TYPE_CODE[qkv.dtype], self._stream())
+        return q, k, v
+
+    def rope_inplace(self, x, positions, cos, sin):
+        self._check("x", x, self._FLOATS, ndim=3)
+        T, heads, hd = x.shape
+        self._check("positions", positions, torch.int32, shape=(T,))
+        self._check("cos", cos, torch.float32, ndim=2)
+        self._check("sin", sin, torch.float32, shape=cos.shape)
+        if hd % 2 or cos.shape[1] != hd // 2:
+            raise ValueError(f"rotary table has {cos.shape[1]} columns for head_dim {hd}")
+        self._call(self.lib.ts_rope_inplace, _ptr(x), _TYPE_CODE[x.dtype], _ptr(positions),
+                   _ptr(cos), _ptr(sin), T, heads, hd, self._stream())
+
+    def kv_store(self, k, v, batch, table, cache):
+        self._check("k", k, self._FLOATS, ndim=3)
+        self._check("v", v, k.dtype, shape=k.shape)
+        T, nkv, hd = k.shape
+        self._check_cache(cache, table, batch, nkv, hd)
+        self._check("positions", batch.positions, torch.int32, shape=(T,))
+        self._call(self.lib.ts_kv_store, _ptr(k), _ptr(v), _TYPE_CODE[k.dtype],
+                   _ptr(cache.k_pages), _ptr(cache.v_pages), _TYPE_CODE[cache.k_pages.dtype],
+                   _ptr(batch.positions), _ptr(batch.entry_of_token), _ptr(table),
+                   table.shape[1], T, nkv, hd, cache.page_size, self._stream())
+
+    # ------------------------------------------------------------ attention
+    def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
+                        scale, window):
+        T = q.shape[0]
+        self._check("q", q, self._FLOATS, shape=(T, num_heads, head_dim))
+        self._check_cache(cache, table, batch, num_kv_heads, head_dim)
+        if T != batch.num_tokens:
+            raise ValueError("q rows differ from the batch's tokens")
+        out = torch.empty_like(q)
+        a = AttentionArgs()
+        a.q, a.out = q.data_ptr(), out.data_ptr()
+        a.k_pages, a.v_pages = cache.k_pages.data_ptr(), cache.v_pages.data_ptr()
+        a.positions, a.entry_of_token = batch.positions.data_ptr(), batch.entry_of_token.data_ptr()
+        a.q_start, a.ctx_len = batch.q_start.data_ptr(), batch.ctx_len.data_ptr()
+        a.table, a.table_width = table.data_ptr(), table.shape[1]
+        a.num_tokens, a.num_entries = T, batch.num_entries
+        a.nq, a.nkv, a.hd = num_heads, num_kv_heads, head_dim
+        a.page_size, a.num_pages = cache.page_size, cache.num_pages
+        a.window = 0 if window is None else int(window)
+        a.scale = scale
+        self._call(self.lib.ts_attention_generic, byref(a), _TYPE_CODE[q.dtype],
+                   _TYPE_CODE[cache.k_pages.dtype], self._stream())
+        return out
+
+    # ------------------------------------------------------------ sampling
+    def argmax(self, logits):
+        self._check("logits", logits, torch.float32, ndim=2)
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        self._call(self.lib.ts_argmax, _ptr(logits), _ptr(out), logits.shape[0],
+                   logits.shape[1], self._stream())
+        return out
+
+    def sample(self, logits, temperatures, keys):
+        """Row r: greedy if temperatures[r] <= 1e-10, else a draw from
+        softmax(logits[r] / T) with noise keyed by keys[r] (int64 bit pattern)."""
+        self._check("logits", logits, torch.float32, ndim=2)
+        R = logits.shape[0]
+        self._check("temperatures", temperatures, torch.float32, shape=(R,))
+        self._check("keys", keys, torch.int64, shape=(R,))
+        out = torch.empty(R, dtype=torch.int32, device=self.device)
+        self._call(self.lib.ts_sample, _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(out),
+                   R, logits.shape[1], self._stream())
+        return out
