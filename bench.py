@@ -1,0 +1,189 @@
+"""Decode and prefill throughput at the Qwen3-0.6B shape with random weights.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the engine (schedule, run, sample, postprocess) for a batch
+of 8 requests with 512-token prompts; `value` is decoded tokens per second.  The same
+line carries a 2,048-token prefill, decode at batch 1 and 64, and the decode step's
+fraction of the HBM roofline.  Peaks are MI355X's published ones.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+
+def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, model=None):
+    import torch
+    from tokensprint_amd.config import Config
+    from tokensprint_amd.engine.assemble import random_model
+    from tokensprint_amd.engine.llm_engine import LLMEngine
+    import tempfile
+    if model is None:
+        cfg = dict(raw)
+        cfg["num_hidden_layers"] = layers
+        _, model = random_model(cfg, seed, dtype, "cuda:0")
+    pages = batch * (-(-max_len // page_size) + 1)
+    config = Config(model=tempfile.gettempdir(), max_model_len=max_len, dtype=model.ctx.dtype,
+                    kvcache_block_size=page_size, num_kvcache_blocks=pages,
+                    max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
+                    chunked_prefill=True, eos=-1)
+    return model, LLMEngine(model, config)
+
+
+def weight_bytes(model) -> int:
+    """Bytes of every weight a decode step reads once (a tied head is counted once;
+    of the embedding table only the head's use is counted when tied)."""
+    seen, total = set(), 0
+    for block in model.blocks:
+        for t in (block.mixer.w_qkv, block.mixer.w_o, block.mixer.w_qnorm, block.mixer.w_knorm,
+                  block.feed_forward.w_gate_up, block.feed_forward.w_down,
+                  block.mixer_norm.weight, block.ffn_norm.weight):
+            if t is not None and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+    for t in (model.head.weight, model.final_norm.weight):
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    return total
+
+
+def decode_run(engine, batch, prompt_len, steps, warmup, vocab):
+    """Prefill `batch` prompts, then time exactly `steps` decode steps."""
+    import torch
+    from tokensprint_amd.config import SamplingParams
+    g = torch.Generator().manual_seed(0)
+    params = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True)
+    for _ in range(batch):
+        engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(), params)
+    while any(r.num_completion_tokens == 0 for r in engine.requests.values()):
+        engine.step()                      # prefill portions until every request has a token
+    for _ in range(warmup):
+        engine.step()
+    ctx0 = sum(len(r) for r in engine.requests.values())
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx1 = sum(len(r) for r in engine.requests.values())
+    # drop the requests
+    for r in list(engine.scheduler.running):
+        engine.scheduler.manager.free(r.cache)
+    engine.scheduler.running.clear()
+    engine.requests.clear()
+    return dt, (ctx0 + ctx1) / 2.0
+
+
+def prefill_run(engine, tokens, vocab, reps=5):
+    import torch
+    from tokensprint_amd.config import SamplingParams
+    g = torch.Generator().manual_seed(1)
+    times = []
+    for _ in range(reps + 1):
+        engine.add_request(torch.randint(0, vocab, (tokens,), generator=g).tolist(),
+                           SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    times = sorted(times[1:])
+    return times[len(times) // 2]
+
+
+def prefill_flops(cfg, layers, T) -> float:
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nq, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_token = 2 * H * (nq + 2 * nkv) * hd + 2 * nq * hd * H + 3 * 2 * H * I
+    attn = 2 * 2 * nq * hd * T * (T + 1) / 2            # causal QK^T and PV
+    return layers * (per_token * T + attn) + 2 * H * V   # head for the last token only
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--model", default="qwen3-0.6b")
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--skip-points", action="store_true", help="only the headline decode run")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+    from tokensprint_amd.config import load_named_config
+
+    raw = load_named_config(args.model)
+    full_layers = raw["num_hidden_layers"]
+    layers = args.layers or full_layers
+    ctx_len, page = 4096, 16
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    item = 2 if dt_name == "bf16" else 4
+    vocab = raw["vocab_size"]
+
+    model, engine = make_engine(raw, args.dtype, layers, args.batch, ctx_len, 2048, page)
+    wbytes = weight_bytes(model)
+    kv_per_token = 2 * layers * raw["num_key_value_heads"] * raw["head_dim"] * item
+
+    dt, mean_tokens = decode_run(engine, args.batch, args.prompt_len, args.steps, args.warmup,
+                                 vocab)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = wbytes + kv_per_token * mean_tokens
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+
+    out = {
+        "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape, 512-token prompts)",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dt_name,
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02) seed 0",
+        "config": {
+            "model": args.model, "global_batch": args.batch, "seq_len": ctx_len,
+            "parallelism": "single-gpu", "layers": layers, "layers_of_model": full_layers,
+            "hidden_size": raw["hidden_size"], "num_heads": raw["num_attention_heads"],
+            "num_kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
+            "intermediate_size": raw["intermediate_size"], "vocab_size": vocab,
+            "tied_embeddings": raw["tie_word_embeddings"], "prompt_len": args.prompt_len,
+            "page_size": page, "mean_context": round(mean_tokens / args.batch, 1),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+
+    if not args.skip_points:
+        T = 2048
+        _, pre_engine = make_engine(raw, args.dtype, layers, 1, ctx_len, T, page, model=model)
+        sec = prefill_run(pre_engine, T, vocab)
+        flops = prefill_flops(raw, layers, T)
+        out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
+                          "frac": round(flops / sec / (MFMA_PEAK_TFLOPS[dt_name] * 1e12), 4)}
+        del pre_engine
+        points = {}
+        for b, steps in ((1, 128), (64, 128)):
+            _, e = make_engine(raw, args.dtype, layers, b, ctx_len, 2048, page, model=model)
+            d, _ = decode_run(e, b, args.prompt_len, steps, 8, vocab)
+            points[f"decode_b{b}"] = round(b * steps / d, 1)
+            del e
+            torch.cuda.empty_cache()
+        out["points"] = points
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -57,6 +57,7 @@ def random_model(raw_config: dict, seed: int, dtype="bfloat16", device="cuda:0",
     """A model with random weights made directly in memory (no folder is written)."""
     from tokensprint_amd.weights.random_init import random_tensors
     config, model = build_model(raw_config, dtype, device, ops)
-    tensors = random_tensors(raw_config, seed, dtype=model.ctx.dtype, std=std)
+    tensors = random_tensors(raw_config, seed, dtype=model.ctx.dtype, std=std,
+                             device=model.ctx.device)
     load_weights(model, TensorDict(tensors), model.ctx.dtype, model.ctx.device)
     return config, model

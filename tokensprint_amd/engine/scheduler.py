@@ -53,12 +53,11 @@ class Scheduler:
                 "Sequence length exceeds max_model_len: "
                 f"got {len(req)}, max allowed is {self.max_model_len - 1}.")
         need = -(-(len(req) + 1) // self.manager.page_size)
-        smallest = min(pool.num_pages for pool in self.manager.pools) \
-            if self.manager.pools else need
-        full_groups = [g for g in self.manager.groups if g.window is None]
-        if full_groups and need > smallest:
+        full = [pool.num_pages for g, pool in zip(self.manager.groups, self.manager.pools)
+                if g.window is None]
+        if full and need > min(full):
             raise ValueError(
-                f"request of {len(req)} tokens needs {need} pages, the pool has {smallest}")
+                f"request of {len(req)} tokens needs {need} pages, the pool has {min(full)}")
         if not self.enable_chunked and len(req) > self.max_num_batched_tokens:
             raise ValueError(
                 f"prompt of {len(req)} tokens exceeds max_num_batched_tokens="
