@@ -34,6 +34,9 @@ class TorchOps:
     def linear(self, x, weight, out_dtype):
         return (x.float() @ weight.float().T).to(out_dtype)
 
+    def linear_silu_mul(self, x, weight, out_dtype):
+        return self.silu_mul(self.linear(x, weight, out_dtype))
+
     def silu_mul(self, gate_up):
         inner = gate_up.shape[-1] // 2
         g, u = gate_up[:, :inner].float(), gate_up[:, inner:].float()
@@ -75,7 +78,7 @@ class TorchOps:
         if (page < 0).any():
             raise RuntimeError("store to a position whose page was given back")
         cache.k_pages[page, :, pos % P] = k.to(cache.k_pages.dtype)
-        cache.v_pages[page, :, pos % P] = v.to(cache.v_pages.dtype)
+        cache.v_pages[page, :, :, pos % P] = v.to(cache.v_pages.dtype)
 
     def qk_norm_rope_store(self, qkv, batch, table, cache, *, num_heads, num_kv_heads,
                            head_dim, q_weight, k_weight, eps, cos_sin):
@@ -109,7 +112,7 @@ class TorchOps:
             if (pages < 0).any():
                 raise RuntimeError("attention reads a position whose page was given back")
             k = cache.k_pages[pages, :, keys % P].float()       # [n, nkv, hd]
-            v = cache.v_pages[pages, :, keys % P].float()
+            v = cache.v_pages[pages, :, :, keys % P].float()
             for j in range(num_heads):
                 s = (k[:, j // group] @ q[t, j].float()) * scale
                 out[t, j] = torch.softmax(s, dim=0) @ v[:, j // group]

@@ -93,6 +93,39 @@ def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
     torch.testing.assert_close(out.double(), ref, **t)
 
 
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (8, 1024, 3072),
+                                   (17, 1000, 2048), (64, 6144, 1024), (3, 151936, 1024),
+                                   (130, 389, 96), (33, 50, 520), (70, 20000, 64)])
+def test_linear_bf16_matrix_core_shapes(ops, gpu_device, out_dtype, M, N, K):
+    x = rand((M, K), torch.bfloat16, gpu_device, 17)
+    w = rand((N, K), torch.bfloat16, gpu_device, 18, scale=0.05)
+    out = ops.linear(x, w, out_dtype)
+    ref = x.float() @ w.float().T
+    t = dict(rtol=2e-3, atol=2e-3) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(out.float(), ref, **t)
+    # a row does not depend on the rest of the batch
+    one = ops.linear(x[M // 2:M // 2 + 1].contiguous(), w, out_dtype)
+    assert torch.equal(out[M // 2:M // 2 + 1], one)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 160, 96), (40, 112, 80), (70, 1000, 520)])
+def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
+    x = rand((M, K), dtype, gpu_device, 19)
+    w = rand((2 * I, K), dtype, gpu_device, 20, scale=0.1)
+    out = ops.linear_silu_mul(x, w, dtype)
+    if dtype == torch.float32:
+        # float64 reference; float32 sums of K products err by about K * 2^-24 * |x||w|
+        gu = x.double() @ w.double().T
+        ref = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+        bound = 1e-5 * float(ref.abs().max())
+        torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=bound)
+    else:
+        ref = REF.linear_silu_mul(x, w, dtype)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):
     x = rand((70, 200), torch.float32, gpu_device, 9)
     w = rand((150, 200), torch.float32, gpu_device, 10)
@@ -160,7 +193,8 @@ def test_rope_reference_shape(ops, gpu_device, dtype):
 
 
 ATTN_SHAPES = [(4, 2, 16, 4), (8, 2, 32, 16), (6, 3, 48, 8), (16, 8, 128, 16), (5, 5, 80, 3),
-               (8, 1, 64, 64), (4, 4, 256, 16), (14, 2, 112, 32)]
+               (8, 1, 64, 64), (4, 4, 256, 16), (14, 2, 112, 32), (32, 1, 64, 16),
+               (40, 2, 32, 8), (3, 1, 96, 12)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -175,6 +209,31 @@ def test_paged_attention(ops, gpu_device, dtype, nq, nkv, hd, page, window):
     out = ops.paged_attention(q, batch, table, cache, **kw)
     ref = REF.paged_attention(q, batch, table, cache, **kw)
     torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 300])
+def test_paged_attention_long_contexts(ops, gpu_device, dtype, window):
+    """Contexts of many key chunks: decode tokens beside a long portion, so both the
+    walk over chunks and the split over waves with its merge are used."""
+    nq, nkv, hd, page = 16, 8, 128, 16
+    for spans in ([(1500, 1), (129, 1), (0, 1)], [(900, 200), (1030, 1)], [(2047, 1)] * 3):
+        batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd,
+                                                page_size=page, spans=spans, seed=31)
+        q = rand((batch.num_tokens, nq, hd), dtype, gpu_device, 32)
+        kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
+        out = ops.paged_attention(q, batch, table, cache, **kw)
+        # reference on a sample of tokens (the plain loop is slow)
+        ref = REF.paged_attention(q, batch, table, cache, **kw) if batch.num_tokens < 20 else None
+        if ref is None:
+            pick = [0, 1, 57, 128, 199, 200]
+            import copy
+            sub = copy.copy(batch)
+            sub.positions = batch.positions[pick].contiguous()
+            sub.entry_of_token = batch.entry_of_token[pick].contiguous()
+            ref = REF.paged_attention(q[pick].contiguous(), sub, table, cache, **kw)
+            out = out[pick]
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -194,7 +253,7 @@ def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
                                   head_dim=hd, scale=1.0, window=None)
         for kvh in range(nkv):
             torch.testing.assert_close(out[0, kvh * 2].float(),
-                                       cache.v_pages[phys, kvh, far % page].float(),
+                                       cache.v_pages[phys, kvh, :, far % page].float(),
                                        rtol=2e-2, atol=2e-2)
 
 

@@ -2,8 +2,11 @@
 
 The reference allocates per layer [2, num_blocks, P, nkv, hd]
 (engine/generation/model_runner.py:420-437).  Here each group of runs has one
-tensor [runs, 2, num_pages, nkv, P, hd], so that one key/value head's part of a page is
-contiguous (P*hd elements) for the attention kernels; a run's view is `LayerCache`.
+pair of tensors: keys [runs, num_pages, nkv, P, hd] and values, transposed inside a
+page, [runs, num_pages, nkv, hd, P].  One key/value head's part of a page is contiguous
+in both; keys are contiguous along the head size (the reduction of q.k) and values along
+the positions (the reduction of p.v), which is what the matrix-core kernels read without
+a transpose.  A run's view is `LayerCache`.
 Per-request state of fixed size lives in [num_slots, *shape] tensors, one per run
 that asks for it.
 """
@@ -46,7 +49,7 @@ class LayerCache:
     page_size: int
     num_pages: int
     k_pages: torch.Tensor | None   # [num_pages, nkv, P, hd]
-    v_pages: torch.Tensor | None
+    v_pages: torch.Tensor | None   # [num_pages, nkv, hd, P]
     state: torch.Tensor | None = None   # [num_slots, *shape] for fixed-size state
 
 
@@ -56,17 +59,19 @@ class CacheStorage:
         self.groups, group_of_run = group_runs(needs)
         counts = [num_pages] * len(self.groups) if isinstance(num_pages, int) else list(num_pages)
         self.page_size, self.num_pages, self.num_slots = page_size, counts, num_slots
-        self.tensors = []
+        self.k_tensors, self.v_tensors = [], []
         for g, n in zip(self.groups, counts):
-            self.tensors.append(torch.zeros(
-                len(g.runs), 2, n, g.num_kv_heads, page_size, g.head_dim,
-                dtype=dtype, device=device))
+            self.k_tensors.append(torch.zeros(
+                len(g.runs), n, g.num_kv_heads, page_size, g.head_dim, dtype=dtype, device=device))
+            self.v_tensors.append(torch.zeros(
+                len(g.runs), n, g.num_kv_heads, g.head_dim, page_size, dtype=dtype, device=device))
         self.views: list[LayerCache | None] = []
         for r, need in enumerate(needs):
             if isinstance(need, PagedKVNeed):
                 g = group_of_run[r]
-                t = self.tensors[g][self.groups[g].runs.index(r)]
-                self.views.append(LayerCache(g, page_size, counts[g], t[0], t[1]))
+                i = self.groups[g].runs.index(r)
+                self.views.append(LayerCache(g, page_size, counts[g], self.k_tensors[g][i],
+                                             self.v_tensors[g][i]))
             elif isinstance(need, SlotStateNeed):
                 state = torch.zeros(num_slots, *need.shape, dtype=need.dtype, device=device)
                 self.views.append(LayerCache(-1, page_size, 0, None, None, state))

@@ -6,7 +6,7 @@ struct AttentionArgs {
   const void* q;          // [T, nq, hd]
   void* out;              // [T, nq, hd]
   const void* k_pages;    // [num_pages, nkv, P, hd]
-  const void* v_pages;
+  const void* v_pages;    // [num_pages, nkv, hd, P]: values transposed inside a page
   const int* positions;       // [T]   absolute position of each query token
   const int* entry_of_token;  // [T]   batch entry (row of the block table) of each token
   const int* q_start;         // [B+1] first flat token of each entry

@@ -43,8 +43,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
     if (valid) {
       const int page = table[j / P];
       if (page >= 0) {
-        row = (((int64_t)page * a.nkv + kvh) * P + j % P) * hd;
-        const TC* kr = kp + row;
+        row = ((int64_t)page * a.nkv + kvh) * P * hd + j % P;   // of the value column
+        const TC* kr = kp + ((int64_t)page * a.nkv + kvh) * P * hd + (int64_t)(j % P) * hd;
         float dot = 0.f;
         for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
         s = dot * a.scale;
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
 #pragma unroll
       for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
         const int d = lane + r * kWave;
-        if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vrow + d]), acc[r]);
+        if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vrow + (int64_t)d * P]), acc[r]);
       }
     }
     __builtin_amdgcn_wave_barrier();

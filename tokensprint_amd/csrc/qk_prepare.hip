@@ -7,7 +7,7 @@ struct QkPrepareArgs {
   const void* qkv;       // [T, (nq + 2*nkv) * hd]
   void* q_out;           // [T, nq, hd]
   void* k_dst;           // pages [num_pages, nkv, P, hd], or flat [T, nkv, hd] if !paged
-  void* v_dst;
+  void* v_dst;           // pages [num_pages, nkv, hd, P] (transposed), or flat [T, nkv, hd]
   const float* q_weight; // [hd] or null: no norm
   const float* k_weight;
   const float* cos;      // [max_pos, hd/2] or null: no rotation
@@ -43,14 +43,21 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
 
   // destination row of hd elements
   int64_t dst_off = -1;
+  int v_stride = 1;   // distance between consecutive head elements of a value row
   if (kind == 0) {
     dst_off = ((int64_t)t * a.nq + h) * hd;
   } else {
     const int kvh = kind == 1 ? h - a.nq : h - a.nq - a.nkv;
     if (a.paged) {
       const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
-      if (page >= 0)
-        dst_off = (((int64_t)page * a.nkv + kvh) * a.page_size + pos % a.page_size) * hd;
+      if (page >= 0) {
+        if (kind == 1) {
+          dst_off = (((int64_t)page * a.nkv + kvh) * a.page_size + pos % a.page_size) * hd;
+        } else {
+          dst_off = ((int64_t)page * a.nkv + kvh) * a.page_size * hd + pos % a.page_size;
+          v_stride = a.page_size;
+        }
+      }
     } else {
       dst_off = ((int64_t)t * a.nkv + kvh) * hd;
     }
@@ -59,7 +66,8 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
 
   if (kind == 2) {
     TC* dst = (TC*)a.v_dst + dst_off;
-    for (int i = lane; i < hd; i += kWave) dst[i] = from_f32<TC>(to_f32(src[i]));
+    for (int i = lane; i < hd; i += kWave)
+      dst[(int64_t)i * v_stride] = from_f32<TC>(to_f32(src[i]));
     return;
   }
 
@@ -162,10 +170,11 @@ __global__ void kv_store_kernel(const T* __restrict__ k, const T* __restrict__ v
   const int pos = positions[t];
   const int page = table[(int64_t)entry_of_token[t] * table_width + pos / page_size];
   if (page < 0) return;
-  const int64_t dst = (((int64_t)page * nkv + kvh) * page_size + pos % page_size) * hd;
+  const int64_t head = ((int64_t)page * nkv + kvh) * page_size * hd;
+  const int slot = pos % page_size;
   for (int i = lane; i < hd; i += kWave) {
-    k_pages[dst + i] = from_f32<TC>(to_f32(k[item * hd + i]));
-    v_pages[dst + i] = from_f32<TC>(to_f32(v[item * hd + i]));
+    k_pages[head + (int64_t)slot * hd + i] = from_f32<TC>(to_f32(k[item * hd + i]));
+    v_pages[head + (int64_t)i * page_size + slot] = from_f32<TC>(to_f32(v[item * hd + i]));
   }
 }
 

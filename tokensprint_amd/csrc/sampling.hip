@@ -22,21 +22,38 @@ __device__ __forceinline__ Best better(Best a, Best b) {
   return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
 }
 
+constexpr int kSlice = 4096;   // vocabulary entries one workgroup scans
+
+__device__ __forceinline__ Best block_best(Best best, float* sv, int* si) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1)
+    best = better(best, Best{__shfl_xor(best.v, o, kWave), __shfl_xor(best.i, o, kWave)});
+  const int wave = threadIdx.x / kWave;
+  if (threadIdx.x % kWave == 0) { sv[wave] = best.v; si[wave] = best.i; }
+  __syncthreads();
+  Best b{sv[0], si[0]};
+  for (int w = 1; w < (int)(blockDim.x / kWave); ++w) b = better(b, Best{sv[w], si[w]});
+  return b;
+}
+
+// Stage 1: workgroup (row, slice) finds the best entry of its slice of the vocabulary.
 template <bool NOISE>
-__global__ __launch_bounds__(256) void pick_kernel(const float* __restrict__ logits,
-                                                   const float* __restrict__ temperature,
-                                                   const uint64_t* __restrict__ keys,
-                                                   int* __restrict__ out, int vocab) {
+__global__ __launch_bounds__(256) void pick_slices_kernel(const float* __restrict__ logits,
+                                                          const float* __restrict__ temperature,
+                                                          const uint64_t* __restrict__ keys,
+                                                          float* __restrict__ part_v,
+                                                          int* __restrict__ part_i, int vocab) {
   __shared__ float sv[4];
   __shared__ int si[4];
-  const int r = blockIdx.x;
+  const int r = blockIdx.x, slice = blockIdx.y;
   const float* row = logits + (int64_t)r * vocab;
   const float temp = NOISE ? temperature[r] : 1.f;
   const bool noisy = NOISE && temp > 1e-10f;
   const float inv_t = noisy ? 1.f / temp : 1.f;
   const uint64_t key = NOISE ? keys[r] : 0;
   Best best{-INFINITY, 0x7fffffff};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+  const int end = min(vocab, (slice + 1) * kSlice);
+  for (int i = slice * kSlice + threadIdx.x; i < end; i += blockDim.x) {
     float s = row[i];
     if (noisy) {
       const float e = fmaxf(-logf(uniform01(key, (uint32_t)i)), 1e-10f);
@@ -44,36 +61,55 @@ __global__ __launch_bounds__(256) void pick_kernel(const float* __restrict__ log
     }
     best = better(best, Best{s, i});
   }
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1)
-    best = better(best, Best{__shfl_xor(best.v, o, kWave), __shfl_xor(best.i, o, kWave)});
-  const int wave = threadIdx.x / kWave;
-  if (threadIdx.x % kWave == 0) { sv[wave] = best.v; si[wave] = best.i; }
-  __syncthreads();
+  best = block_best(best, sv, si);
   if (threadIdx.x == 0) {
-    Best b{sv[0], si[0]};
-    for (int w = 1; w < 4; ++w) b = better(b, Best{sv[w], si[w]});
-    out[r] = b.i;
+    part_v[(int64_t)r * gridDim.y + slice] = best.v;
+    part_i[(int64_t)r * gridDim.y + slice] = best.i;
   }
 }
 
-extern "C" int ts_argmax(const float* logits, int* out, int rows, int vocab,
-                         hipStream_t stream) {
+// Stage 2: one workgroup per row picks among the slices' winners.
+__global__ __launch_bounds__(256) void pick_final_kernel(const float* __restrict__ part_v,
+                                                         const int* __restrict__ part_i,
+                                                         int* __restrict__ out, int slices) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  const int r = blockIdx.x;
+  Best best{-INFINITY, 0x7fffffff};
+  for (int i = threadIdx.x; i < slices; i += blockDim.x)
+    best = better(best, Best{part_v[(int64_t)r * slices + i], part_i[(int64_t)r * slices + i]});
+  best = block_best(best, sv, si);
+  if (threadIdx.x == 0) out[r] = best.i;
+}
+
+extern "C" int ts_pick_slices(int vocab) { return (vocab + kSlice - 1) / kSlice; }
+
+// `part_v` / `part_i`: scratch of rows * ts_pick_slices(vocab) entries each.
+extern "C" int ts_argmax(const float* logits, int* out, float* part_v, int* part_i, int rows,
+                         int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) TS_FAIL("argmax: vocab=%d", vocab);
-  hipLaunchKernelGGL(pick_kernel<false>, dim3(rows), dim3(256), 0, stream, logits,
-                     (const float*)nullptr, (const uint64_t*)nullptr, out, vocab);
+  const int slices = (vocab + kSlice - 1) / kSlice;
+  hipLaunchKernelGGL(pick_slices_kernel<false>, dim3(rows, slices), dim3(256), 0, stream,
+                     logits, (const float*)nullptr, (const uint64_t*)nullptr, part_v, part_i,
+                     vocab);
+  hipLaunchKernelGGL(pick_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out,
+                     slices);
   TS_CHECK_LAUNCH("argmax");
   return 0;
 }
 
 // temperature[r] <= 1e-10 means greedy for that row.
 extern "C" int ts_sample(const float* logits, const float* temperature, const uint64_t* keys,
-                         int* out, int rows, int vocab, hipStream_t stream) {
+                         int* out, float* part_v, int* part_i, int rows, int vocab,
+                         hipStream_t stream) {
   if (rows <= 0) return 0;
   if (vocab <= 0) TS_FAIL("sample: vocab=%d", vocab);
-  hipLaunchKernelGGL(pick_kernel<true>, dim3(rows), dim3(256), 0, stream, logits, temperature,
-                     keys, out, vocab);
+  const int slices = (vocab + kSlice - 1) / kSlice;
+  hipLaunchKernelGGL(pick_slices_kernel<true>, dim3(rows, slices), dim3(256), 0, stream, logits,
+                     temperature, keys, part_v, part_i, vocab);
+  hipLaunchKernelGGL(pick_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out,
+                     slices);
   TS_CHECK_LAUNCH("sample");
   return 0;
 }

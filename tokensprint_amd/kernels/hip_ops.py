@@ -34,6 +34,10 @@ class QkPrepareArgs(Structure):
     ]
 
 
+class AttentionMfmaArgs(Structure):
+    pass
+
+
 class AttentionArgs(Structure):
     _fields_ = [
         ("q", c_void_p), ("out", c_void_p), ("k_pages", c_void_p), ("v_pages", c_void_p),
@@ -43,6 +47,13 @@ class AttentionArgs(Structure):
         ("nkv", c_int), ("hd", c_int), ("page_size", c_int), ("num_pages", c_int),
         ("window", c_int), ("scale", c_float),
     ]
+
+
+AttentionMfmaArgs._fields_ = [
+    ("base", AttentionArgs), ("tiles", c_void_p), ("partial_o", c_void_p),
+    ("partial_ml", c_void_p), ("num_tiles", c_int), ("rows_per_token", c_int),
+    ("head_blocks", c_int), ("num_splits", c_int),
+]
 
 
 def _load_library() -> ctypes.CDLL:
@@ -70,6 +81,7 @@ class HipOps:
             raise KernelError(
                 "the HIP kernels need an AMD GPU (device 'cuda:N'); there is no CPU path")
         self.lib = _load_library()
+        self._attn_chunk = self.lib.ts_attention_mfma_chunk()
 
     # ------------------------------------------------------------ helpers
     def _stream(self):
@@ -154,10 +166,36 @@ class HipOps:
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
-        self._call(self.lib.ts_gemm_fma, _ptr(x), _TYPE_CODE[x.dtype], _ptr(weight),
-                   _TYPE_CODE[weight.dtype], _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
-                   self._stream())
+        if self._mfma_ok(x, weight):
+            self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
+                       _TYPE_CODE[out_dtype], M, N, K, 0, self._stream())
+        else:
+            self._call(self.lib.ts_gemm_fma, _ptr(x), _TYPE_CODE[x.dtype], _ptr(weight),
+                       _TYPE_CODE[weight.dtype], _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                       self._stream())
         return out
+
+    @staticmethod
+    def _mfma_ok(x, weight):
+        """The matrix-core product takes bfloat16 operands with K a multiple of 8;
+        everything else (float32 anywhere) goes to the float32 multiply-add kernel."""
+        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and x.shape[1] % 8 == 0)
+
+    def linear_silu_mul(self, x, weight, out_dtype):
+        """silu(x Wg^T) * (x Wu^T) for weight = [Wg; Wu] stacked by rows -> [M, N/2]."""
+        self._check("x", x, self._FLOATS, ndim=2)
+        self._check("weight", weight, self._FLOATS, ndim=2)
+        M, K = x.shape
+        if weight.shape[1] != K or weight.shape[0] % 2:
+            raise ValueError(f"linear_silu_mul: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
+        inner = weight.shape[0] // 2
+        if self._mfma_ok(x, weight) and out_dtype == torch.bfloat16:
+            out = torch.empty(M, inner, dtype=out_dtype, device=self.device)
+            self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
+                       _TYPE_CODE[out_dtype], M, inner, K, 1, self._stream())
+            return out
+        return self.silu_mul(self.linear(x, weight, out_dtype))
 
     # ------------------------------------------------------------ q/k preparation
     def _qk_args(self, qkv, batch, *, num_heads, kv_in_row, head_dim, q_weight, k_weight, eps,
@@ -197,7 +235,8 @@ class HipOps:
         P = cache.page_size
         self._check("k_pages", cache.k_pages, self._FLOATS,
                     shape=(cache.num_pages, nkv, P, head_dim))
-        self._check("v_pages", cache.v_pages, cache.k_pages.dtype, shape=cache.k_pages.shape)
+        self._check("v_pages", cache.v_pages, cache.k_pages.dtype,
+                    shape=(cache.num_pages, nkv, head_dim, P))
         self._check("block table", table, torch.int32, ndim=2)
         if table.shape[0] != batch.num_entries:
             raise ValueError("block table rows differ from the batch's entries")
@@ -277,6 +316,53 @@ class HipOps:
             raise ValueError("q rows differ from the batch's tokens")
         out = torch.empty_like(q)
         a = AttentionArgs()
+        self._fill_attention_args(a, q, out, batch, table, cache, num_heads, num_kv_heads,
+                                  head_dim, scale, window)
+        if (q.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
+                and head_dim % 16 == 0 and head_dim <= 256 and cache.page_size % 4 == 0):
+            self._attention_mfma(a, batch, num_heads // num_kv_heads)
+        else:
+            self._call(self.lib.ts_attention_generic, byref(a), _TYPE_CODE[q.dtype],
+                       _TYPE_CODE[cache.k_pages.dtype], self._stream())
+        return out
+
+    def _attention_mfma(self, a, batch, group):
+        """Tile the batch's queries (16 rows of q heads x tokens per wavefront), choose how
+        many waves share a tile's keys, and launch."""
+        rows_per_token = min(group, 16)
+        head_blocks = -(-group // 16)
+        tokens_per_tile = 16 // rows_per_token
+        key = ("attn_tiles", tokens_per_tile)
+        if key not in batch.plans:
+            tiles = []
+            first = 0
+            for entry, n in enumerate(batch.q_lens):
+                for t0 in range(0, n, tokens_per_tile):
+                    tiles.append((entry, first + t0, min(tokens_per_tile, n - t0)))
+                first += n
+            host = torch.tensor(tiles, dtype=torch.int32)
+            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
+        tiles_dev, num_tiles = batch.plans[key]
+        items = num_tiles * a.nkv * head_blocks
+        chunk = self._attn_chunk
+        span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
+                                                           a.window + batch.max_q_len + chunk)
+        max_chunks = max(1, -(-span // chunk))
+        splits = min(max_chunks, max(1, 2048 // items))
+        m = AttentionMfmaArgs()
+        m.base = a
+        m.tiles = tiles_dev.data_ptr()
+        m.num_tiles, m.rows_per_token, m.head_blocks = num_tiles, rows_per_token, head_blocks
+        m.num_splits = splits
+        if splits > 1:
+            po = torch.empty(items * splits * 16 * a.hd, dtype=torch.float32, device=self.device)
+            pml = torch.empty(items * splits * 16 * 2, dtype=torch.float32, device=self.device)
+            m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
+        self._call(self.lib.ts_attention_mfma, byref(m), self._stream())
+
+    def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
+                             head_dim, scale, window):
+        T = q.shape[0]
         a.q, a.out = q.data_ptr(), out.data_ptr()
         a.k_pages, a.v_pages = cache.k_pages.data_ptr(), cache.v_pages.data_ptr()
         a.positions, a.entry_of_token = batch.positions.data_ptr(), batch.entry_of_token.data_ptr()
@@ -287,17 +373,21 @@ class HipOps:
         a.page_size, a.num_pages = cache.page_size, cache.num_pages
         a.window = 0 if window is None else int(window)
         a.scale = scale
-        self._call(self.lib.ts_attention_generic, byref(a), _TYPE_CODE[q.dtype],
-                   _TYPE_CODE[cache.k_pages.dtype], self._stream())
-        return out
 
     # ------------------------------------------------------------ sampling
     def argmax(self, logits):
         self._check("logits", logits, torch.float32, ndim=2)
-        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
-        self._call(self.lib.ts_argmax, _ptr(logits), _ptr(out), logits.shape[0],
-                   logits.shape[1], self._stream())
+        R, V = logits.shape
+        out = torch.empty(R, dtype=torch.int32, device=self.device)
+        part_v, part_i = self._pick_scratch(R, V)
+        self._call(self.lib.ts_argmax, _ptr(logits), _ptr(out), _ptr(part_v), _ptr(part_i), R, V,
+                   self._stream())
         return out
+
+    def _pick_scratch(self, rows, vocab):
+        slices = self.lib.ts_pick_slices(vocab)
+        return (torch.empty(rows * slices, dtype=torch.float32, device=self.device),
+                torch.empty(rows * slices, dtype=torch.int32, device=self.device))
 
     def sample(self, logits, temperatures, keys):
         """Row r: greedy if temperatures[r] <= 1e-10, else a draw from
@@ -307,6 +397,7 @@ class HipOps:
         self._check("temperatures", temperatures, torch.float32, shape=(R,))
         self._check("keys", keys, torch.int64, shape=(R,))
         out = torch.empty(R, dtype=torch.int32, device=self.device)
+        part_v, part_i = self._pick_scratch(R, logits.shape[1])
         self._call(self.lib.ts_sample, _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(out),
-                   R, logits.shape[1], self._stream())
+                   _ptr(part_v), _ptr(part_i), R, logits.shape[1], self._stream())
         return out

@@ -1,6 +1,7 @@
 """Dense SwiGLU feed-forward: down(silu(gate(h)) * up(h)), no bias
 (engine/nn/layers.py:61-66).  Gate and up run as one product over row-concatenated
-weights; the activation kernel reads both halves."""
+weights, with the activation applied as the product is written where the kernel
+can, and by a separate kernel over both halves otherwise."""
 
 from __future__ import annotations
 
@@ -34,6 +35,5 @@ class SwiGLU(FeedForward):
         self.w_down = get(pre + "down_proj.weight")
 
     def forward(self, h, batch):
-        gu = self.ops.linear(h, self.w_gate_up, self.ctx.dtype)
-        act = self.ops.silu_mul(gu)
+        act = self.ops.linear_silu_mul(h, self.w_gate_up, self.ctx.dtype)
         return self.ops.linear(act, self.w_down, self.ctx.dtype)
