@@ -63,3 +63,48 @@ def test_mixed_with_page_reuse(setup):
     runner = runner_for(model, page, 224 // page)      # 261 tokens in all: pages are reused
     drives.compare(drives.drive_mixed(runner, requests), ref, rtol, atol)
     assert all(pool.num_used == 0 for pool in runner.manager.pools)
+
+
+def test_captured_decode_steps(setup):
+    """Decode through captured graphs: every replay is checked against the plain logits,
+    with eager steps (another request's prompt) between replays and two bucket sizes."""
+    from tokensprint_amd.engine import StepEntry
+    model, page, requests, ref, (rtol, atol) = setup
+    runner = ModelRunner(model, page_size=page, num_pages=320 // page, num_slots=4,
+                         graph_max_len=128)
+    col = drives.Collector()
+    ids = ["r3", "r4", "r7"]
+    live = {}
+    for rid in ids:
+        rc = runner.manager.admit(rid)
+        head = len(requests[rid]) - 30
+        runner.manager.extend(rc, head)
+        e = [StepEntry(rc, requests[rid][:head], 0, list(range(head)))]
+        col.take(e, runner.step(e))
+        live[rid] = [rc, head]
+    for step in range(30):
+        entries = []
+        for rid in (ids if step % 3 else ids[:2]):          # buckets of 4 and of 2
+            rc, pos = live[rid]
+            if pos >= len(requests[rid]):
+                continue
+            runner.manager.extend(rc, pos + 1)
+            entries.append(StepEntry(rc, requests[rid][pos:pos + 1], pos, [0]))
+            live[rid][1] = pos + 1
+        assert runner._graph_bucket(entries) in (2, 4)
+        col.take(entries, runner.step(entries).clone())
+        if step % 5 == 0:                                     # eager work between replays
+            rc = runner.manager.admit("other")
+            runner.manager.extend(rc, 17)
+            runner.step([StepEntry(rc, requests["r2"], 0, [16])])
+            runner.manager.free(rc)
+    assert set(runner.graphs) == {2, 4}
+    # finish the requests eagerly where steps were skipped
+    for rid in ids:
+        rc, pos = live[rid]
+        while pos < len(requests[rid]):
+            runner.manager.extend(rc, pos + 1)
+            e = [StepEntry(rc, requests[rid][pos:pos + 1], pos, [0])]
+            col.take(e, runner.step(e).clone())
+            pos += 1
+    drives.compare(col, {rid: ref[rid] for rid in ids}, rtol, atol)

@@ -31,9 +31,13 @@ struct AttentionMfmaArgs {
   int rows_per_token;    // query heads of a tile per token: min(group, 16)
   int head_blocks;       // ceil(group / 16)
   int num_splits;
+  int cooperative;       // 1: a workgroup per item (few tiles), 0: a wavefront per item
 };
 
-template <int HD>
+// COOP = false: a wavefront per item walks its keys alone (many tiles: prompts).
+// COOP = true: a workgroup per item; its four waves take every fourth 32-key block and
+// merge in LDS (few tiles: decode), so a short context costs one round of loads.
+template <int HD, bool COOP>
 __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs args) {
   constexpr int KS = (HD + 31) / 32;   // k-steps of the first product over the head size
   constexpr int DB = HD / 16;          // 16-row blocks of O^T
@@ -42,7 +46,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   const int r = lane % 16, g = lane / 16;
   const int group = a.nq / a.nkv;
   const int items = args.num_tiles * a.nkv * args.head_blocks;
-  const int item = blockIdx.x * 4 + wave;
+  const int item = COOP ? blockIdx.x : blockIdx.x * 4 + wave;
   if (item >= items) return;
   const int tile = item / (a.nkv * args.head_blocks);
   const int kvh = (item / args.head_blocks) % a.nkv;
@@ -68,9 +72,8 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   const int c_first = lo_tile / kChunk, c_last = pos_last / kChunk;
   const int per = (c_last - c_first + args.num_splits) / args.num_splits;   // ceil(n / splits)
   const int c0 = c_first + split * per, c1 = min(c0 + per, c_last + 1);
-
   if (c0 > c_last) {   // more splits than chunks: a neutral partial, no data touched
-    if (g == 0) {
+    if (g == 0 && (!COOP || wave == 0)) {
       const int64_t slot = ((int64_t)item * args.num_splits + split) * 16 + r;
       args.partial_ml[slot * 2] = -INFINITY;
       args.partial_ml[slot * 2 + 1] = 0.f;
@@ -80,6 +83,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
 
   // Q^T operand: lane (r, g) holds Q[row r][g*8*KS + s*8 + j]
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16x4 zero4 = {0, 0, 0, 0};
   bf16x8 qv[KS];
   {
     const bf16_t* q = (const bf16_t*)a.q + ((int64_t)token * a.nq + head) * HD;
@@ -97,24 +101,52 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   const bf16_t* kp = (const bf16_t*)a.k_pages;
   const bf16_t* vp = (const bf16_t*)a.v_pages;
 
-  const int key_begin = max(c0 * kChunk, lo_tile & ~31);
+  const int key_begin = max(c0 * kChunk, lo_tile & ~31) + (COOP ? wave * 32 : 0);
   const int key_end = min(c1 * kChunk, pos_last + 1);
-  for (int kb = key_begin; kb < key_end; kb += 32) {
-    // ---- S^T for 32 keys: two blocks of 16
-    f32x4 st[2];
+  constexpr int kStride = COOP ? 128 : 32;
+
+  // K operand of a 32-key block: lane (r, g) holds K[key blk*16 + r][g*8*KS + s*8 + j]
+  bf16x8 kv[2][KS];
+  auto load_k = [&](int kb) {
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
-      st[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
       const int key = kb + blk * 16 + r;
       const int page = key <= pos_last ? table[key / P] : -1;
       const bf16_t* krow = kp + (((int64_t)max(page, 0) * a.nkv + kvh) * P + key % P) * HD;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const int e = g * 8 * KS + s * 8;
-        const bf16x8 kv = (page >= 0 && e < HD) ? *(const bf16x8*)(krow + e) : zero8;
-        st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, qv[s], st[blk], 0, 0, 0);
+        kv[blk][s] = (page >= 0 && e < HD) ? *(const bf16x8*)(krow + e) : zero8;
       }
     }
+  };
+  if (key_begin < key_end) load_k(key_begin);
+
+  for (int kb = key_begin; kb < key_end; kb += kStride) {
+    // ---- V^T operand of this block, asked for before the scores are worked out.
+    //      Slot (g, j) of the reduction stands for key kb + g*4 + j (j < 4) or
+    //      kb + 16 + g*4 + j - 4, in both operands of the second product.
+    bf16x4 vv[2][DB];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int key4 = kb + blk * 16 + g * 4;
+      const int page = key4 <= pos_last ? table[key4 / P] : -1;
+      const bf16_t* vcol = vp + ((int64_t)max(page, 0) * a.nkv + kvh) * HD * P + key4 % P;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        vv[blk][db] = page >= 0 ? *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P) : zero4;
+    }
+    // ---- S^T for 32 keys: two blocks of 16
+    f32x4 st[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      st[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv[blk][s], qv[s], st[blk], 0, 0, 0);
+    }
+    // ---- keys of the next block, in flight during the softmax and the second product
+    if (kb + kStride < key_end) load_k(kb + kStride);
     // ---- mask, running maximum and sum of my query (column r; lanes r, r+16, r+32, r+48)
     float sv[8];
     float mx = -INFINITY;
@@ -145,28 +177,53 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
     ps += __shfl_xor(ps, 32, kWave);
     l = l * corr + ps;
     m = m_new;
-    // ---- O^T += V^T P^T.  Slot (g, j) of the reduction stands for key
-    //      kb + g*4 + j (j < 4) or kb + 16 + g*4 + j - 4, in both operands.
-    const bf16_t* vcol[2];
-    bool v_ok[2];
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      const int key4 = kb + blk * 16 + g * 4;
-      const int page = key4 <= pos_last ? table[key4 / P] : -1;
-      v_ok[blk] = page >= 0;
-      vcol[blk] = vp + ((int64_t)max(page, 0) * a.nkv + kvh) * HD * P + key4 % P;
-    }
+    // ---- O^T += V^T P^T
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      const bf16x4 z4 = {0, 0, 0, 0};
-      const int d = db * 16 + r;
-      const bf16x4 v0 = v_ok[0] ? *(const bf16x4*)(vcol[0] + (int64_t)d * P) : z4;
-      const bf16x4 v1 = v_ok[1] ? *(const bf16x4*)(vcol[1] + (int64_t)d * P) : z4;
-      const bf16x8 vv = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      const bf16x4 v0 = vv[0][db], v1 = vv[1][db];
+      const bf16x8 vfull = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       f32x4 acc = o[db];
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[t] *= corr;
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pv, acc, 0, 0, 0);
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfull, pv, acc, 0, 0, 0);
+    }
+  }
+
+  if (COOP) {   // the four waves' partial results, merged by wave 0 in wave order
+    __shared__ float s_ml[3][kWave][2];
+    __shared__ f32x4 s_o[3][DB][kWave];
+    if (wave > 0) {
+      s_ml[wave - 1][lane][0] = m;
+      s_ml[wave - 1][lane][1] = l;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) s_o[wave - 1][db][lane] = o[db];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float M = m;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) M = fmaxf(M, s_ml[w][lane][0]);
+    if (M != -INFINITY) {
+      const float w0 = __expf(m - M);
+      l *= w0;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) o[db][t] *= w0;
+#pragma unroll
+      for (int w = 0; w < 3; ++w) {
+        const float mw = s_ml[w][lane][0];
+        if (mw == -INFINITY) continue;
+        const float ww = __expf(mw - M);
+        l += s_ml[w][lane][1] * ww;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const f32x4 ow = s_o[w][db][lane];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) o[db][t] += ow[t] * ww;
+        }
+      }
+      m = M;
     }
   }
 
@@ -183,9 +240,11 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
     }
   } else {
     const int64_t slot = ((int64_t)item * args.num_splits + split) * 16 + r;
-    float* po = args.partial_o + slot * HD;
+    if (row_ok) {
+      float* po = args.partial_o + slot * HD;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) *(f32x4*)(po + db * 16 + g * 4) = o[db];
+      for (int db = 0; db < DB; ++db) *(f32x4*)(po + db * 16 + g * 4) = o[db];
+    }
     if (g == 0) {
       args.partial_ml[slot * 2] = m;
       args.partial_ml[slot * 2 + 1] = l;
@@ -208,12 +267,18 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
   const int ti = r / args.rows_per_token, hh = hb * 16 + r % args.rows_per_token;
   if (ti >= ntok || hh >= group) return;
   const int64_t base = (int64_t)item * args.num_splits * 16 + r;
+  // splits beyond the tile's chunks hold nothing: same arithmetic as the first kernel
+  const int pos_first = a.positions[tok0], pos_last = a.positions[tok0 + ntok - 1];
+  const int lo_tile = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+  const int nchunks = pos_last / kChunk - lo_tile / kChunk + 1;
+  const int per = (nchunks - 1 + args.num_splits) / args.num_splits;
+  const int used = min(args.num_splits, (nchunks + per - 1) / per);
   float M = -INFINITY;
-  for (int s = 0; s < args.num_splits; ++s)
+  for (int s = 0; s < used; ++s)
     M = fmaxf(M, args.partial_ml[(base + (int64_t)s * 16) * 2]);
   float L = 0.f;
   float acc[HD / 16] = {};
-  for (int s = 0; s < args.num_splits; ++s) {
+  for (int s = 0; s < used; ++s) {
     const int64_t slot = base + (int64_t)s * 16;
     const float ms = args.partial_ml[slot * 2];
     if (ms == -INFINITY) continue;
@@ -233,8 +298,13 @@ int ts_check_attention_args(const AttentionArgs& a, const char* who);
 template <int HD>
 static int launch_mfma(const AttentionMfmaArgs& args, hipStream_t stream) {
   const int items = args.num_tiles * args.base.nkv * args.head_blocks;
-  dim3 grid((items + 3) / 4, args.num_splits);
-  hipLaunchKernelGGL(attention_mfma_kernel<HD>, grid, dim3(256), 0, stream, args);
+  if (args.cooperative) {
+    hipLaunchKernelGGL((attention_mfma_kernel<HD, true>), dim3(items, args.num_splits),
+                       dim3(256), 0, stream, args);
+  } else {
+    hipLaunchKernelGGL((attention_mfma_kernel<HD, false>), dim3((items + 3) / 4, args.num_splits),
+                       dim3(256), 0, stream, args);
+  }
   if (args.num_splits > 1)
     hipLaunchKernelGGL(attention_merge_kernel<HD>, dim3(items), dim3(256), 0, stream, args);
   return 0;

@@ -54,6 +54,68 @@ def _align(n: int, a: int = 4) -> int:
     return -(-n // a) * a
 
 
+def decode_layout(bucket: int, widths: list[int]):
+    """Section offsets of a decode-only batch of `bucket` entries, one token each."""
+    sizes = [bucket, bucket, bucket, bucket + 1, bucket, bucket, bucket] \
+        + [bucket * w for w in widths]
+    offs, total = [], 0
+    for n in sizes:
+        offs.append(total)
+        total += _align(n)
+    return offs, total
+
+
+class StaticDecodeBatch:
+    """A decode batch of fixed size in fixed device memory, for a captured graph.
+
+    `fill` rewrites the contents for the step's entries; lanes beyond them are idle:
+    token 0 at position 0 with no pages, so they write nothing to the cache
+    (as the reference pads with slot -1, engine/generation/model_runner.py:253-276).
+    """
+
+    def __init__(self, device, bucket: int, widths: list[int]) -> None:
+        self.bucket, self.widths = bucket, widths
+        self.offs, total = decode_layout(bucket, widths)
+        self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=device)
+        self.copied = torch.cuda.Event()
+        o, B = self.offs, bucket
+        d = self.dev
+        self.batch = StepBatch(
+            num_tokens=B, num_entries=B, num_logit_rows=B,
+            token_ids=d[o[0]:o[0] + B], positions=d[o[1]:o[1] + B],
+            entry_of_token=d[o[2]:o[2] + B], q_start=d[o[3]:o[3] + B + 1],
+            ctx_len=d[o[4]:o[4] + B], slot_ids=d[o[5]:o[5] + B], logit_rows=d[o[6]:o[6] + B],
+            tables=[d[o[7 + g]:o[7 + g] + B * w].view(B, w) for g, w in enumerate(widths)],
+            q_lens=[1] * B, starts=[0] * B, max_q_len=1, max_ctx_len=0)
+        h = self.host.numpy()
+        h[:] = 0
+        h[o[2]:o[2] + B] = np.arange(B)
+        h[o[3]:o[3] + B + 1] = np.arange(B + 1)
+        h[o[6]:o[6] + B] = np.arange(B)
+
+    def fill(self, entries) -> None:
+        o, B, n = self.offs, self.bucket, len(entries)
+        self.copied.synchronize()          # the last copy out of the pinned buffer is done
+        h = self.host.numpy()
+        h[o[0]:o[0] + B] = 0
+        h[o[1]:o[1] + B] = 0
+        h[o[4]:o[4] + B] = 1
+        h[o[5]:o[5] + B] = 0
+        h[o[0]:o[0] + n] = [e.tokens[0] for e in entries]
+        h[o[1]:o[1] + n] = [e.start for e in entries]
+        h[o[4]:o[4] + n] = [e.start + 1 for e in entries]
+        h[o[5]:o[5] + n] = [e.cache.slot for e in entries]
+        for g, w in enumerate(self.widths):
+            tab = h[o[7 + g]:o[7 + g] + B * w].reshape(B, w)
+            tab[:] = -1
+            for i, e in enumerate(entries):
+                t = e.cache.tables[g]
+                tab[i, :len(t)] = t
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+
 class BatchBuilder:
     """Packs a step's description into one pinned buffer and one device copy."""
 
@@ -64,12 +126,16 @@ class BatchBuilder:
         self.vocab_size = vocab_size
         self.max_position = max_position
         self._pinned = None
+        self._copied = None
 
     def _host_buffer(self, n: int) -> torch.Tensor:
         if self.device.type != "cuda":
             return torch.empty(n, dtype=torch.int32)
         if self._pinned is None or self._pinned.numel() < n:
             self._pinned = torch.empty(max(n, 1 << 16), dtype=torch.int32, pin_memory=True)
+            self._copied = torch.cuda.Event()
+        else:
+            self._copied.synchronize()     # the last copy out of the pinned buffer is done
         return self._pinned[:n]
 
     def build(self, entries: list[StepEntry], table_width: list[int] | None = None) -> StepBatch:
@@ -133,8 +199,11 @@ class BatchBuilder:
                 tab[i, :len(t)] = t
             buf[offs[7 + g]:offs[7 + g] + B * w] = tab.reshape(-1)
 
-        dev = host.to(self.device, non_blocking=True) if self.device.type == "cuda" \
-            else host.clone()
+        if self.device.type == "cuda":
+            dev = host.to(self.device, non_blocking=True)
+            self._copied.record()
+        else:
+            dev = host.clone()
 
         def sec(i, n):
             return dev[offs[i]:offs[i] + n]

@@ -34,8 +34,10 @@ class LLMEngine:
         if num_pages < 0:
             num_pages = self._pages_from_free_memory(model, config)
             config.num_kvcache_blocks = num_pages
-        self.runner = ModelRunner(model, page_size=page, num_pages=num_pages,
-                                  num_slots=config.max_num_seqs)
+        self.runner = ModelRunner(
+            model, page_size=page, num_pages=num_pages, num_slots=config.max_num_seqs,
+            graph_max_len=None if config.enforce_eager or model.ctx.device.type != "cuda"
+            else config.max_model_len)
         self.scheduler = Scheduler(
             self.runner.manager, max_num_batched_tokens=config.max_num_batched_tokens,
             max_num_seqs=config.max_num_seqs, max_model_len=config.max_model_len,

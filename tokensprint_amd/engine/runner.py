@@ -12,13 +12,16 @@ from __future__ import annotations
 import torch
 
 from tokensprint_amd.cache import CacheManager, CacheStorage, page_bytes
-from tokensprint_amd.engine.batch import BatchBuilder, StepBatch, StepEntry
+from tokensprint_amd.engine.batch import BatchBuilder, StaticDecodeBatch, StepBatch, StepEntry
 from tokensprint_amd.models.model import Model
 
 
 class ModelRunner:
     def __init__(self, model: Model, *, page_size: int, num_pages: int, num_slots: int,
-                 cache_dtype: torch.dtype | None = None) -> None:
+                 cache_dtype: torch.dtype | None = None, graph_max_len: int | None = None,
+                 graph_max_batch: int = 256) -> None:
+        """`graph_max_len`: the longest request a captured decode graph must serve (its
+        block tables are that wide); None means every step runs eagerly."""
         self.model = model
         self.device = model.ctx.device
         self.dtype = model.ctx.dtype
@@ -30,6 +33,11 @@ class ModelRunner:
                                     vocab_size=model.spec.vocab_size,
                                     max_position=model.spec.max_position)
         self.page_size = page_size
+        self.graph_max_len = graph_max_len
+        self.graphs: dict[int, tuple] = {}      # bucket -> (graph, static batch, logits)
+        top = min(graph_max_batch, num_slots)
+        self.buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, top + 1, 16)) + [top]
+                               if b <= top}) if graph_max_len else []
 
     @staticmethod
     def pages_that_fit(model: Model, page_size: int, free_bytes: int,
@@ -50,4 +58,50 @@ class ModelRunner:
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Logits float32 [sum(len(e.want)), vocab], in the order of entries and want."""
+        bucket = self._graph_bucket(entries)
+        if bucket is not None:
+            return self._replay(bucket, entries)
         return self.run(self.build(entries))
+
+    # ------------------------------------------------------------ captured decode steps
+    # The reference captures model.decode for decode-only batches per batch-size bucket
+    # and runs head and sampler eagerly (engine/generation/model_runner.py:203-390);
+    # here the captured region also holds the head, and buckets are captured at first use.
+    def _graph_bucket(self, entries):
+        if not self.buckets or len(entries) > self.buckets[-1]:
+            return None
+        for e in entries:
+            if len(e.tokens) != 1 or e.want != [0] or e.start + 1 > self.graph_max_len:
+                return None
+        return next(b for b in self.buckets if b >= len(entries))
+
+    def _capture(self, bucket: int):
+        widths = [-(-self.graph_max_len // self.page_size)] * len(self.storage.groups)
+        static = StaticDecodeBatch(self.device, bucket, widths)
+        static.batch.max_ctx_len = self.graph_max_len
+        static.fill([])
+        torch.cuda.synchronize(self.device)
+        side = torch.cuda.Stream(self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):          # loads kernels, fills the batch's launch plans
+            self.run(static.batch)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.run(static.batch)
+        self.graphs[bucket] = (graph, static, logits)
+        return self.graphs[bucket]
+
+    def _replay(self, bucket: int, entries: list[StepEntry]) -> torch.Tensor:
+        graph, static, logits = self.graphs.get(bucket) or self._capture(bucket)
+        vocab = self.model.spec.vocab_size
+        for e in entries:
+            if not 0 <= e.tokens[0] < vocab:
+                raise ValueError(f"token id {e.tokens[0]} outside [0, {vocab})")
+            if e.start + 1 > e.cache.num_tokens:
+                raise ValueError(f"request {e.cache.request_id!r}: position {e.start} is not "
+                                 "covered by its cache")
+        static.fill(entries)
+        graph.replay()
+        return logits[:len(entries)]

@@ -52,7 +52,7 @@ class AttentionArgs(Structure):
 AttentionMfmaArgs._fields_ = [
     ("base", AttentionArgs), ("tiles", c_void_p), ("partial_o", c_void_p),
     ("partial_ml", c_void_p), ("num_tiles", c_int), ("rows_per_token", c_int),
-    ("head_blocks", c_int), ("num_splits", c_int),
+    ("head_blocks", c_int), ("num_splits", c_int), ("cooperative", c_int),
 ]
 
 
@@ -348,8 +348,12 @@ class HipOps:
         span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
                                                            a.window + batch.max_q_len + chunk)
         max_chunks = max(1, -(-span // chunk))
-        splits = min(max_chunks, max(1, 2048 // items))
+        # few tiles (decode): a workgroup per tile and chunk, its waves share the chunk;
+        # many tiles (prompts): a wavefront per tile walks its keys
+        cooperative = items <= 1024
+        splits = min(max_chunks, max(1, (1024 if cooperative else 4096) // items))
         m = AttentionMfmaArgs()
+        m.cooperative = int(cooperative)
         m.base = a
         m.tiles = tiles_dev.data_ptr()
         m.num_tiles, m.rows_per_token, m.head_blocks = num_tiles, rows_per_token, head_blocks
