@@ -34,6 +34,14 @@ class TorchOps:
     def linear(self, x, weight, out_dtype):
         return (x.float() @ weight.float().T).to(out_dtype)
 
+    def norm_linear(self, resid, delta, norm_weight, eps, weight, out_dtype, silu_mul=False):
+        act = torch.bfloat16 if weight.dtype == torch.bfloat16 else torch.float32
+        h = self.rmsnorm(resid, norm_weight, eps, act) if delta is None \
+            else self.add_rmsnorm(resid, delta, norm_weight, eps, act)
+        out = self.linear_silu_mul(h, weight, out_dtype) if silu_mul \
+            else self.linear(h, weight, out_dtype)
+        return out, resid
+
     def linear_silu_mul(self, x, weight, out_dtype):
         return self.silu_mul(self.linear(x, weight, out_dtype))
 

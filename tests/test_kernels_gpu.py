@@ -126,6 +126,25 @@ def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("M,N,K", [(8, 4096, 1024), (1, 160, 96), (16, 112, 80), (3, 1024, 3072),
+                                   (20, 96, 64), (5, 20000, 64)])
+def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
+    resid = rand((M, K), torch.float32, gpu_device, 40)
+    delta = rand((M, K), dtype, gpu_device, 41)
+    nw = 1 + 0.1 * rand((K,), torch.float32, gpu_device, 42)
+    w = rand((N, K), dtype, gpu_device, 43, scale=0.05)
+    for d in (delta, None):
+        r_ref = resid.clone()
+        ref, r_ref = REF.norm_linear(r_ref, d, nw, 1e-5, w, dtype, silu_mul=silu)
+        r_in = resid.clone()
+        out, r_out = ops.norm_linear(r_in, d, nw, 1e-5, w, dtype, silu_mul=silu)
+        torch.testing.assert_close(r_out, r_ref, rtol=0, atol=0)
+        t = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
+        torch.testing.assert_close(out.float(), ref.float(), **t)
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):
     x = rand((70, 200), torch.float32, gpu_device, 9)
     w = rand((150, 200), torch.float32, gpu_device, 10)
@@ -234,6 +253,28 @@ def test_paged_attention_long_contexts(ops, gpu_device, dtype, window):
             ref = REF.paged_attention(q[pick].contiguous(), sub, table, cache, **kw)
             out = out[pick]
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("window", [None, 100])
+@pytest.mark.parametrize("nq,nkv,hd,page", [(16, 8, 128, 16), (8, 2, 64, 16), (6, 3, 48, 8),
+                                            (4, 4, 256, 32), (32, 1, 32, 16)])
+def test_paged_attention_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
+    """Portions long enough for the multi-tile prompt kernel (bfloat16), with and without
+    cached context before them, beside a decode token."""
+    dtype = torch.bfloat16
+    spans = [(0, 700), (333, 1), (50, 515)]
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=33)
+    q = rand((batch.num_tokens, nq, hd), dtype, gpu_device, 34)
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
+    out = ops.paged_attention(q, batch, table, cache, **kw)
+    pick = [0, 1, 7, 8, 15, 16, 31, 32, 33, 255, 256, 699, 700, 701, 702, 709, 900, 1215]
+    import copy
+    sub = copy.copy(batch)
+    sub.positions = batch.positions[pick].contiguous()
+    sub.entry_of_token = batch.entry_of_token[pick].contiguous()
+    ref = REF.paged_attention(q[pick].contiguous(), sub, table, cache, **kw)
+    torch.testing.assert_close(out[pick].float(), ref.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1,0 +1,200 @@
+// The inner work of the matrix-core attention kernels: operand loads for a block of 32
+// keys and the update of one 16-row query tile with that block.
+//
+// Layouts (v_mfma_f32_16x16x32_bf16, lane = 16*g + r):
+//   K operand   lane (r, g) holds K[key blk*16 + r][g*8*KS + s*8 + j]        (A of S^T = K Q^T)
+//   Q operand   lane (r, g) holds Q[row r][g*8*KS + s*8 + j]                 (B)
+//   S^T result  lane (r, g) holds S^T[key blk*16 + g*4 + t][row r]
+//   V operand   lane (r, g) holds V^T[d = db*16 + r][keys blk0: g*4..+3, blk1: g*4..+3]
+//   P operand   lane (r, g) holds its own 8 probabilities, in that key order
+// so a lane's scores are, in place, its part of the second product's B operand, and the
+// softmax statistics of a query row live in the four lanes r, r+16, r+32, r+48.
+//
+// PAGE16: the page size is a multiple of 16, so a block of 16 keys lies in one page and
+// its page id is the same for the whole wave: the ids come out of a register strip of
+// the block table by readlane, addresses are scalar plus a lane offset, and all loads
+// of a block are independent of each other.  Otherwise every lane looks its page up
+// (small test page sizes; slow but the same arithmetic).
+#pragma once
+#include "attention_mfma.h"
+
+template <int HD>
+struct KvBlock {
+  static constexpr int KS = (HD + 31) / 32;
+  static constexpr int DB = HD / 16;
+  bf16x8 k[2][KS];
+  bf16x4 v[2][DB];
+};
+
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// Page ids of the coming 32-key block, fetched one block ahead through the scalar cache
+// (read-only, wave-uniform addresses), so that neither a wait for vector loads nor an
+// address dependency stands between a block's loads.
+typedef const int __attribute__((address_space(4))) * ConstTable;
+
+struct PageCursor {
+  ConstTable table;   // block table row of the entry
+  int page_size;
+  int last_key;
+  int next[2];        // page ids of the two 16-key blocks of the next call
+  __device__ __forceinline__ int fetch(int k0) const {          // k0 is wave-uniform
+    return k0 <= last_key ? table[k0 / page_size] : -1;
+  }
+  __device__ __forceinline__ void start(int kb) {
+    next[0] = fetch(kb);
+    next[1] = fetch(kb + 16);
+  }
+};
+
+// Loads the K and V operands of keys [kb, kb + 32).  With PAGE16 calls must come in
+// steps of `stride` keys from the cursor's start (the cursor holds this call's pages and
+// then fetches those of kb + stride).
+template <int HD, bool PAGE16>
+__device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArgs& a,
+                                              const int* table, PageCursor& cur, int kvh,
+                                              int kb, int stride, int r, int g) {
+  constexpr int KS = KvBlock<HD>::KS, DB = KvBlock<HD>::DB;
+  const bf16_t* kp = (const bf16_t*)a.k_pages;
+  const bf16_t* vp = (const bf16_t*)a.v_pages;
+  const int P = a.page_size;
+  const int last_key = cur.last_key;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const int k0 = kb + blk * 16;                        // first key of the 16-key block
+    if (PAGE16) {
+      const int page = cur.next[blk];                    // scalar
+      if (page >= 0) {
+        const int off = k0 % P;
+        const bf16_t* krow = kp + (((int64_t)page * a.nkv + kvh) * P + off + r) * HD;
+        const bf16_t* vcol = vp + ((int64_t)page * a.nkv + kvh) * HD * P + off + g * 4;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const int e = g * 8 * KS + s * 8;
+          b.k[blk][s] = (KS * 32 == HD || e < HD) ? *(const bf16x8*)(krow + e) : zero8;
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          b.v[blk][db] = *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P);
+      } else {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) b.k[blk][s] = zero8;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) b.v[blk][db] = zero4;
+      }
+    } else {
+      const int key = k0 + r;
+      const int kpage = key <= last_key ? table[key / P] : -1;
+      const bf16_t* krow = kp + (((int64_t)max(kpage, 0) * a.nkv + kvh) * P + key % P) * HD;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int e = g * 8 * KS + s * 8;
+        b.k[blk][s] = (kpage >= 0 && e < HD) ? *(const bf16x8*)(krow + e) : zero8;
+      }
+      const int key4 = k0 + g * 4;
+      const int vpage = key4 <= last_key ? table[key4 / P] : -1;
+      const bf16_t* vcol = vp + ((int64_t)max(vpage, 0) * a.nkv + kvh) * HD * P + key4 % P;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        b.v[blk][db] = vpage >= 0 ? *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P) : zero4;
+    }
+  }
+  if (PAGE16) cur.start(kb + stride);
+}
+
+// One query tile's running state.
+template <int HD>
+struct TileState {
+  static constexpr int KS = (HD + 31) / 32;
+  static constexpr int DB = HD / 16;
+  bf16x8 q[KS];
+  f32x4 o[DB];
+  float m, l;
+  int pos, lo;        // this lane's row: position and first visible key (pos = -1: no row)
+};
+
+template <int HD>
+__device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow, bool row_ok,
+                                           int g) {
+  constexpr int KS = TileState<HD>::KS;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int e = g * 8 * KS + s * 8;
+    t.q[s] = (row_ok && e < HD) ? *(const bf16x8*)(qrow + e) : zero8;
+  }
+#pragma unroll
+  for (int db = 0; db < TileState<HD>::DB; ++db) t.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  t.m = -INFINITY;
+  t.l = 0.f;
+}
+
+// Scores of the block for one tile, masked softmax update, and O^T += V^T P^T.
+// `interior`: every key of the block is visible to every row of the tile (wave-uniform),
+// so the mask is skipped.  scale_log2 = softmax scale * log2(e); m is kept in that unit.
+template <int HD>
+__device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>& b, int kb,
+                                            float scale_log2, bool interior, int g) {
+  constexpr int KS = TileState<HD>::KS, DB = TileState<HD>::DB;
+  f32x4 st[2];
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    st[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+      st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[blk][s], t.q[s], st[blk], 0, 0, 0);
+  }
+  float sv[8];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float s = st[blk][i] * scale_log2;
+      if (!interior) {
+        const int key = kb + blk * 16 + g * 4 + i;
+        s = (key <= t.pos && key >= t.lo) ? s : -INFINITY;
+      }
+      sv[blk * 4 + i] = s;
+      mx = fmaxf(mx, s);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  const float m_new = fmaxf(t.m, mx);
+  const bool any = m_new != -INFINITY;
+  const float corr = any ? __builtin_amdgcn_exp2f(t.m - m_new) : 1.f;
+  float ps = 0.f;
+  bf16x8 pv;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float p = any ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.f;
+    ps += p;
+    pv[i] = (bf16_t)p;
+  }
+  ps += __shfl_xor(ps, 16, kWave);
+  ps += __shfl_xor(ps, 32, kWave);
+  t.l = t.l * corr + ps;
+  t.m = m_new;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    const bf16x4 v0 = b.v[0][db], v1 = b.v[1][db];
+    const bf16x8 vfull = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+    f32x4 acc = t.o[db];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= corr;
+    t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfull, pv, acc, 0, 0, 0);
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void store_tile(const TileState<HD>& t, bf16_t* out, int g) {
+  const float inv = t.l > 0.f ? 1.f / t.l : 0.f;
+#pragma unroll
+  for (int db = 0; db < TileState<HD>::DB; ++db) {
+    bf16x4 ov = {(bf16_t)(t.o[db][0] * inv), (bf16_t)(t.o[db][1] * inv),
+                 (bf16_t)(t.o[db][2] * inv), (bf16_t)(t.o[db][3] * inv)};
+    *(bf16x4*)(out + db * 16 + g * 4) = ov;
+  }
+}

@@ -53,6 +53,7 @@ AttentionMfmaArgs._fields_ = [
     ("base", AttentionArgs), ("tiles", c_void_p), ("partial_o", c_void_p),
     ("partial_ml", c_void_p), ("num_tiles", c_int), ("rows_per_token", c_int),
     ("head_blocks", c_int), ("num_splits", c_int), ("cooperative", c_int),
+    ("tiles_per_wave", c_int),
 ]
 
 
@@ -165,6 +166,8 @@ class HipOps:
         N = weight.shape[0]
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
+        if self._library_ok(x, weight, out_dtype):
+            return torch.matmul(x, weight.t())
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         if self._mfma_ok(x, weight):
             self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
@@ -175,12 +178,59 @@ class HipOps:
                        self._stream())
         return out
 
+    # Rows from which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
+    # torch.matmul), as the reference sends every linear layer to its vendor library
+    # (engine/nn/base_layers.py:7-10).  Below it the weight-streaming kernels are faster.
+    LIBRARY_ROWS = 192
+
+    @classmethod
+    def _library_ok(cls, x, weight, out_dtype):
+        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and out_dtype == torch.bfloat16 and x.shape[0] >= cls.LIBRARY_ROWS)
+
     @staticmethod
     def _mfma_ok(x, weight):
         """The matrix-core product takes bfloat16 operands with K a multiple of 8;
         everything else (float32 anywhere) goes to the float32 multiply-add kernel."""
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and x.shape[1] % 8 == 0)
+
+    def norm_linear(self, resid, delta, norm_weight, eps, weight, out_dtype, silu_mul=False):
+        """(RMSNorm(resid + delta) W^T, resid + delta): the residual add, the norm and
+        the product in one kernel where it can be (bfloat16 weights, at most 16 rows);
+        otherwise the same from separate kernels.  `delta` may be None.  With `silu_mul`
+        the weight is [Wg; Wu] and the result silu(h Wg^T) * (h Wu^T).  The returned
+        residual stream may or may not be the tensor passed in."""
+        self._check("resid", resid, torch.float32, ndim=2)
+        M, K = resid.shape
+        self._check("weight", weight, self._FLOATS, ndim=2)
+        if weight.shape[1] != K:
+            raise ValueError(f"norm_linear: stream width {K}, weight has {weight.shape[1]} columns")
+        fused = (weight.dtype == torch.bfloat16 and M <= 16 and K % 8 == 0
+                 and M * (K + 8) * 2 <= 140 * 1024
+                 and (out_dtype == torch.bfloat16 or not silu_mul)
+                 and out_dtype in (torch.bfloat16, torch.float32))
+        if not fused:
+            act = torch.bfloat16 if weight.dtype == torch.bfloat16 else torch.float32
+            h = self.rmsnorm(resid, norm_weight, eps, act) if delta is None \
+                else self.add_rmsnorm(resid, delta, norm_weight, eps, act)
+            out = self.linear_silu_mul(h, weight, out_dtype) if silu_mul \
+                else self.linear(h, weight, out_dtype)
+            return out, resid
+        self._check("norm weight", norm_weight, torch.float32, shape=(K,))
+        if delta is not None:
+            self._check("delta", delta, self._FLOATS, shape=resid.shape)
+        N = weight.shape[0] // 2 if silu_mul else weight.shape[0]
+        if silu_mul and weight.shape[0] % 2:
+            raise ValueError("norm_linear: stacked gate/up weight needs an even row count")
+        out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        resid_out = torch.empty_like(resid)
+        self._call(self.lib.ts_norm_gemm_mfma_bf16, _ptr(resid), _ptr(delta),
+                   _TYPE_CODE[delta.dtype] if delta is not None else 0,
+                   1 if delta is not None else 0, _ptr(norm_weight), c_float(eps),
+                   _ptr(resid_out), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                   int(silu_mul), self._stream())
+        return out, resid_out
 
     def linear_silu_mul(self, x, weight, out_dtype):
         """silu(x Wg^T) * (x Wu^T) for weight = [Wg; Wu] stacked by rows -> [M, N/2]."""
@@ -190,7 +240,8 @@ class HipOps:
         if weight.shape[1] != K or weight.shape[0] % 2:
             raise ValueError(f"linear_silu_mul: x {tuple(x.shape)}, weight {tuple(weight.shape)}")
         inner = weight.shape[0] // 2
-        if self._mfma_ok(x, weight) and out_dtype == torch.bfloat16:
+        if (self._mfma_ok(x, weight) and out_dtype == torch.bfloat16
+                and not self._library_ok(x, weight, out_dtype)):
             out = torch.empty(M, inner, dtype=out_dtype, device=self.device)
             self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
                        _TYPE_CODE[out_dtype], M, inner, K, 1, self._stream())
@@ -332,17 +383,19 @@ class HipOps:
         rows_per_token = min(group, 16)
         head_blocks = -(-group // 16)
         tokens_per_tile = 16 // rows_per_token
-        key = ("attn_tiles", tokens_per_tile)
-        if key not in batch.plans:
-            tiles = []
-            first = 0
-            for entry, n in enumerate(batch.q_lens):
-                for t0 in range(0, n, tokens_per_tile):
-                    tiles.append((entry, first + t0, min(tokens_per_tile, n - t0)))
-                first += n
-            host = torch.tensor(tiles, dtype=torch.int32)
-            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
-        tiles_dev, num_tiles = batch.plans[key]
+        m = AttentionMfmaArgs()
+        m.base = a
+        m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
+        # long portions of prompts: a wavefront takes several query tiles and walks alone
+        tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
+        if tiles16 * a.nkv * head_blocks >= 2048:
+            tpw = self.lib.ts_attention_prefill_tiles(a.hd)
+            tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw)
+            m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
+            m.num_splits = 1
+            self._call(self.lib.ts_attention_prefill, byref(m), self._stream())
+            return
+        tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile)
         items = num_tiles * a.nkv * head_blocks
         chunk = self._attn_chunk
         span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
@@ -352,17 +405,29 @@ class HipOps:
         # many tiles (prompts): a wavefront per tile walks its keys
         cooperative = items <= 1024
         splits = min(max_chunks, max(1, (1024 if cooperative else 4096) // items))
-        m = AttentionMfmaArgs()
         m.cooperative = int(cooperative)
-        m.base = a
-        m.tiles = tiles_dev.data_ptr()
-        m.num_tiles, m.rows_per_token, m.head_blocks = num_tiles, rows_per_token, head_blocks
+        m.tiles, m.num_tiles = tiles_dev.data_ptr(), num_tiles
         m.num_splits = splits
         if splits > 1:
             po = torch.empty(items * splits * 16 * a.hd, dtype=torch.float32, device=self.device)
             pml = torch.empty(items * splits * 16 * 2, dtype=torch.float32, device=self.device)
             m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
         self._call(self.lib.ts_attention_mfma, byref(m), self._stream())
+
+    def _attention_tiles(self, batch, tokens):
+        """Device list of (entry, first flat token, tokens) cutting every entry of the batch
+        into runs of at most `tokens` consecutive tokens; made once per step and size."""
+        key = ("attn_tiles", tokens)
+        if key not in batch.plans:
+            tiles = []
+            first = 0
+            for entry, n in enumerate(batch.q_lens):
+                for t0 in range(0, n, tokens):
+                    tiles.append((entry, first + t0, min(tokens, n - t0)))
+                first += n
+            host = torch.tensor(tiles, dtype=torch.int32)
+            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
+        return batch.plans[key]
 
     def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
                              head_dim, scale, window):

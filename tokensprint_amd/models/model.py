@@ -87,8 +87,11 @@ class Model:
         if batch.num_logit_rows == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=resid.device)
         resid_rows = ops.gather_rows(resid, batch.logit_rows)
-        if delta is None:
-            h = self.final_norm.forward(resid_rows)
-        else:
-            h = self.final_norm.add_forward(resid_rows, ops.gather_rows(delta, batch.logit_rows))
+        delta_rows = None if delta is None else ops.gather_rows(delta, batch.logit_rows)
+        fused = self.final_norm.fused_rmsnorm()
+        if fused is not None:
+            return ops.norm_linear(resid_rows, delta_rows, fused[0], fused[1], self.head.weight,
+                                   torch.float32)[0]
+        h = self.final_norm.forward(resid_rows) if delta_rows is None \
+            else self.final_norm.add_forward(resid_rows, delta_rows)
         return self.head.forward(h)

@@ -68,14 +68,25 @@ class GroupedQueryAttention(Mixer):
         return PagedKVNeed(self.nkv, self.hd, self.window)
 
     # -- step
+    def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache):
+        fused = norm.fused_rmsnorm()
+        if fused is None:
+            return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache)
+        qkv, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_qkv,
+                                          self.ctx.dtype)
+        return self._attend(qkv, batch, cache, write_cache), resid
+
     def forward(self, h, batch, cache, write_cache):
+        return self._attend(self.ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache,
+                            write_cache)
+
+    def _attend(self, qkv, batch, cache, write_cache):
         if cache is None:
             raise RuntimeError("gqa_attention needs a paged key/value cache")
         if write_cache and not self.own_kv:
             raise RuntimeError(f"{self.prefix}: a layer without k/v weights cannot own a cache")
-        ops, T = self.ops, h.shape[0]
+        ops, T = self.ops, qkv.shape[0]
         nkv_here = self.nkv if self.own_kv else 0
-        qkv = ops.linear(h, self.w_qkv, self.ctx.dtype)
         table = batch.tables[cache.group]
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None

@@ -81,6 +81,11 @@ class Part:
 
 
 class Norm(Part):
+    def fused_rmsnorm(self):
+        """(weight, eps) if this norm is a plain RMSNorm a kernel may fuse into the product
+        that follows it, else None."""
+        return None
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """Normalised copy of x [T, width] in the activation dtype."""
         raise NotImplementedError
@@ -113,10 +118,22 @@ class Mixer(Part):
         """h [T, width] -> [T, width].  `cache` is this run's cache view (or None)."""
         raise NotImplementedError
 
+    def forward_from_stream(self, resid, delta, norm: Norm, batch, cache, write_cache: bool):
+        """The same from the residual stream: adds `delta` (may be None) to `resid`,
+        norms, mixes.  Returns (output, residual stream after the add).  A part overrides
+        this to fuse the add and the norm into its first product."""
+        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
+        return self.forward(h, batch, cache, write_cache), resid
+
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
+
+    def forward_from_stream(self, resid, delta, norm: Norm, batch):
+        """See Mixer.forward_from_stream."""
+        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
+        return self.forward(h, batch), resid
 
 
 class Block:

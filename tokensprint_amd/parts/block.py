@@ -9,9 +9,7 @@ from tokensprint_amd.parts.base import BLOCKS, Block, register
 @register(BLOCKS, "pre_norm")
 class PreNormBlock(Block):
     def forward(self, resid, delta, batch, cache, write_cache):
-        h = self.mixer_norm.forward(resid) if delta is None \
-            else self.mixer_norm.add_forward(resid, delta)
-        a = self.mixer.forward(h, batch, cache, write_cache)
-        h = self.ffn_norm.add_forward(resid, a)
-        f = self.feed_forward.forward(h, batch)
+        a, resid = self.mixer.forward_from_stream(resid, delta, self.mixer_norm, batch, cache,
+                                                  write_cache)
+        f, resid = self.feed_forward.forward_from_stream(resid, a, self.ffn_norm, batch)
         return resid, f
