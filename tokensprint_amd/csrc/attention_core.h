@@ -10,7 +10,7 @@
 // so a lane's scores are, in place, its part of the second product's B operand, and the
 // softmax statistics of a query row live in the four lanes r, r+16, r+32, r+48.
 //
-// PAGE16: the page size is a multiple of 16, so a block of 16 keys lies in one page and
+// PAGE16: the page size is a power of two from 16 up, so a block of 16 keys lies in one page and
 // its page id is the same for the whole wave: the ids come out of a register strip of
 // the block table by readlane, addresses are scalar plus a lane offset, and all loads
 // of a block are independent of each other.  Otherwise every lane looks its page up
@@ -28,6 +28,24 @@ struct KvBlock {
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
+// Reductions over the four lanes r, r+16, r+32, r+48 that share a query row, with the
+// gfx950 row-swap instructions (no LDS round trip): v_permlane16_swap exchanges odd rows
+// of 16 lanes of one operand with even rows of the other, v_permlane32_swap the upper 32
+// lanes of one with the lower 32 of the other; fed the same value twice they return the
+// value of each half (pair of rows) in both halves.
+__device__ __forceinline__ float col4_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float col4_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Page ids of the coming 32-key block, fetched one block ahead through the scalar cache
 // (read-only, wave-uniform addresses), so that neither a wait for vector loads nor an
 // address dependency stands between a block's loads.
@@ -35,15 +53,16 @@ typedef const int __attribute__((address_space(4))) * ConstTable;
 
 struct PageCursor {
   ConstTable table;   // block table row of the entry
-  int page_size;
+  int page_size;      // with PAGE16 a power of two >= 16
   int last_key;
-  int next[2];        // page ids of the two 16-key blocks of the next call
+  int next0, next1;   // page ids of the two 16-key blocks of the next call (two
+                      // scalars: an array indexed at run time would live in memory)
   __device__ __forceinline__ int fetch(int k0) const {          // k0 is wave-uniform
-    return k0 <= last_key ? table[k0 / page_size] : -1;
+    return k0 <= last_key ? table[k0 >> (__builtin_ctz(page_size))] : -1;
   }
   __device__ __forceinline__ void start(int kb) {
-    next[0] = fetch(kb);
-    next[1] = fetch(kb + 16);
+    next0 = fetch(kb);
+    next1 = fetch(kb + 16);
   }
 };
 
@@ -65,9 +84,9 @@ __device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArg
   for (int blk = 0; blk < 2; ++blk) {
     const int k0 = kb + blk * 16;                        // first key of the 16-key block
     if (PAGE16) {
-      const int page = cur.next[blk];                    // scalar
+      const int page = blk ? cur.next1 : cur.next0;      // scalar
       if (page >= 0) {
-        const int off = k0 % P;
+        const int off = k0 & (P - 1);
         const bf16_t* krow = kp + (((int64_t)page * a.nkv + kvh) * P + off + r) * HD;
         const bf16_t* vcol = vp + ((int64_t)page * a.nkv + kvh) * HD * P + off + g * 4;
 #pragma unroll
@@ -160,8 +179,7 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
       sv[blk * 4 + i] = s;
       mx = fmaxf(mx, s);
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  mx = col4_max(mx);
   const float m_new = fmaxf(t.m, mx);
   const bool any = m_new != -INFINITY;
   const float corr = any ? __builtin_amdgcn_exp2f(t.m - m_new) : 1.f;
@@ -173,8 +191,7 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
     ps += p;
     pv[i] = (bf16_t)p;
   }
-  ps += __shfl_xor(ps, 16, kWave);
-  ps += __shfl_xor(ps, 32, kWave);
+  ps = col4_sum(ps);
   t.l = t.l * corr + ps;
   t.m = m_new;
 #pragma unroll

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   constexpr int kStride = COOP ? 128 : 32;
   const int key_begin = max(c0 * kChunk, lo_tile & ~31) + (COOP ? wave * 32 : 0);
   const int key_end = min(c1 * kChunk, pos_last + 1);
-  PageCursor cur{(ConstTable)table, a.page_size, pos_last, {-1, -1}};
+  PageCursor cur{(ConstTable)table, a.page_size, pos_last, -1, -1};
   if (PAGE16) cur.start(key_begin);
 
   KvBlock<HD> A, B;
@@ -191,7 +191,8 @@ int ts_check_attention_args(const AttentionArgs& a, const char* who);
 template <int HD>
 static int launch_mfma(const AttentionMfmaArgs& args, hipStream_t stream) {
   const int items = args.num_tiles * args.base.nkv * args.head_blocks;
-  const bool page16 = args.base.page_size % 16 == 0;
+  const int P = args.base.page_size;
+  const bool page16 = P >= 16 && (P & (P - 1)) == 0;
   const dim3 coop_grid(items, args.num_splits), walk_grid((items + 3) / 4, args.num_splits);
   if (args.cooperative && page16)
     hipLaunchKernelGGL((attention_mfma_kernel<HD, true, true>), coop_grid, dim3(256), 0, stream, args);

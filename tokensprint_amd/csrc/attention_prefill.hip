@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
   }
 
   const int key_begin = lo_all & ~31;
-  PageCursor cur{(ConstTable)table, a.page_size, pos_last, {-1, -1}};
+  PageCursor cur{(ConstTable)table, a.page_size, pos_last, -1, -1};
   if (PAGE16) cur.start(key_begin);
 
   auto work = [&](const KvBlock<HD>& b, int kb) {
@@ -85,10 +85,163 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
   }
 }
 
-// Query tiles per wavefront: as many as the register file holds accumulators for.
-constexpr int tiles_per_wave(int hd) { return hd <= 64 ? 4 : (hd <= 128 ? 2 : 1); }
+// ---------------------------------------------------------------------------------
+// The same walk with the workgroup's four waves sharing every K and V block through LDS
+// (page sizes that are powers of two from 16 up).  The waves take four consecutive query tiles of
+// one entry and one key/value head; per block of 32 keys each wave fetches a quarter of
+// the operand registers from global memory and stores them to LDS in operand layout,
+// double-buffered: the fetch of block i+1 is in flight while block i is worked on, and
+// one barrier per block separates the two.  A block is read from L2 once per workgroup
+// instead of once per wave, and operands come out of LDS just before their product, so
+// few registers are held and several workgroups share a CU.
+template <int HD>
+__global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfmaArgs args) {
+  constexpr int KS = (HD + 31) / 32, DB = HD / 16;
+  constexpr int KQ = (2 * KS + 3) / 4, VQ = (2 * DB + 3) / 4;    // operand slots per wave
+  __shared__ bf16x8 k_lds[2][2 * KS][kWave];
+  __shared__ bf16x4 v_lds[2][2 * DB][kWave];
+  const AttentionArgs& a = args.base;
+  const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int r = lane % 16, g = lane / 16;
+  const int group = a.nq / a.nkv;
+  const int heads = a.nkv * args.head_blocks;
+  const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
+  const int item = args.num_tiles - 1 - blockIdx.x / heads;    // longest key ranges first
+  const int kvh = head_slot / args.head_blocks;
+  const int hb = head_slot % args.head_blocks;
+  const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
+            ntok = uniform(args.tiles[item * 3 + 2]);
+  const int* table = a.table + (int64_t)entry * a.table_width;
+  const int P = a.page_size;
+  const int tq = 16 / args.rows_per_token;
 
-extern "C" int ts_attention_prefill_tiles(int head_dim) { return tiles_per_wave(head_dim); }
+  // this wave's tile: tokens [wave*tq, wave*tq + tq) of the item
+  const int ti = wave * tq + r / args.rows_per_token;
+  const int hh = hb * 16 + r % args.rows_per_token;
+  const int head = kvh * group + min(hh, group - 1);
+  const bool row_ok = ti < ntok && hh < group;
+  const int pos_first = uniform(a.positions[tok0]);
+  const int pos_last = pos_first + ntok - 1;
+  const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+  const float scale_log2 = a.scale * 1.44269504088896341f;
+
+  TileState<HD> t;
+  t.pos = row_ok ? pos_first + ti : -1;
+  t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+  const int tile_first = pos_first + wave * tq;
+  const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
+  const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
+  const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+  load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
+                 row_ok, g);
+
+  const bf16_t* kp = (const bf16_t*)a.k_pages;
+  const bf16_t* vp = (const bf16_t*)a.v_pages;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16x4 zero4 = {0, 0, 0, 0};
+  PageCursor cur{(ConstTable)table, P, pos_last, -1, -1};
+  const int key_begin = lo_all & ~31;
+  cur.start(key_begin);
+
+  // This wave's quarter of a block's operands: global -> registers.  The loads are
+  // issued unconditionally (a missing page reads page 0 and is zeroed when stored to
+  // LDS), so nothing but the barrier stands between them and the work on the block.
+  constexpr bool kEven = (2 * KS) % 4 == 0, vEven = (2 * DB) % 4 == 0;
+  bf16x8 kreg[KQ];
+  bf16x4 vreg[VQ];
+  bool kvalid[KQ], vvalid[VQ];                  // wave-uniform
+  // address = head base + page * page stride (scalar) + position in page (scalar)
+  //           + this lane's offset inside the slot (fixed for the whole walk)
+  const int64_t k_page_stride = (int64_t)a.nkv * P * HD, v_page_stride = k_page_stride;
+  const bf16_t* k_head = kp + (int64_t)kvh * P * HD;
+  const bf16_t* v_head = vp + (int64_t)kvh * HD * P;
+  int k_lane[KQ], v_lane[VQ], k_blk[KQ], v_blk[VQ];
+  bool k_dim_ok[KQ];
+#pragma unroll
+  for (int i = 0; i < KQ; ++i) {
+    const int q = kEven ? wave + 4 * i : min(wave + 4 * i, 2 * KS - 1);
+    const int s0 = q % KS;
+    k_blk[i] = q / KS;
+    k_dim_ok[i] = KS * 32 == HD || g * 8 * KS + s0 * 8 < HD;
+    k_lane[i] = r * HD + min(g * 8 * KS + s0 * 8, HD - 8);
+  }
+#pragma unroll
+  for (int i = 0; i < VQ; ++i) {
+    const int q = vEven ? wave + 4 * i : min(wave + 4 * i, 2 * DB - 1);
+    v_blk[i] = q / DB;
+    v_lane[i] = ((q % DB) * 16 + r) * P + g * 4;
+  }
+  auto fetch = [&](int kb) {
+    const int in_page = kb & (P - 1);             // a block of 16 keys never straddles a page
+    const int page0 = cur.next0, page1 = cur.next1;
+    const bf16_t* kb0 = k_head + (int64_t)max(page0, 0) * k_page_stride + in_page * HD;
+    const bf16_t* kb1 = k_head + (int64_t)max(page1, 0) * k_page_stride +
+                        ((in_page + 16) & (P - 1)) * HD;
+    const bf16_t* vb0 = v_head + (int64_t)max(page0, 0) * v_page_stride + in_page;
+    const bf16_t* vb1 = v_head + (int64_t)max(page1, 0) * v_page_stride + ((in_page + 16) & (P - 1));
+#pragma unroll
+    for (int i = 0; i < KQ; ++i) {
+      kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
+      kreg[i] = *(const bf16x8*)((k_blk[i] ? kb1 : kb0) + k_lane[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VQ; ++i) {
+      vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
+      vreg[i] = *(const bf16x4*)((v_blk[i] ? vb1 : vb0) + v_lane[i]);
+    }
+    cur.start(kb + 32);
+  };
+  auto stash = [&](int buf) {                      // registers -> LDS, operand layout
+#pragma unroll
+    for (int i = 0; i < KQ; ++i)
+      if (kEven || wave + 4 * i < 2 * KS)
+        k_lds[buf][wave + 4 * i][lane] = kvalid[i] ? kreg[i] : zero8;
+#pragma unroll
+    for (int i = 0; i < VQ; ++i)
+      if (vEven || wave + 4 * i < 2 * DB)
+        v_lds[buf][wave + 4 * i][lane] = vvalid[i] ? vreg[i] : zero4;
+  };
+
+  fetch(key_begin);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kb = key_begin; kb <= pos_last; kb += 32, buf ^= 1) {
+    const bool more = kb + 32 <= pos_last;
+    if (more) fetch(kb + 32);
+    if (kb <= tile_last && kb + 31 >= tile_lo) {
+      KvBlock<HD> b;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+#pragma unroll
+        for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = k_lds[buf][blk * KS + s0][lane];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) b.v[blk][db] = v_lds[buf][blk * DB + db][lane];
+      }
+      tile_update<HD>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+  }
+  if (row_ok)
+    store_tile<HD>(t, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+}
+
+// Query tiles per wavefront: as many as the register file holds accumulators for.
+constexpr int tiles_per_wave(int hd) { return hd <= 32 ? 4 : (hd <= 64 ? 2 : 1); }
+
+// Tokens one work item covers, in 16-row tiles: four (one per wave) for the LDS kernel.
+extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size) {
+  return page_size >= 16 && (page_size & (page_size - 1)) == 0 ? 4 : tiles_per_wave(head_dim);
+}
+
+template <int HD>
+static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream) {
+  if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
+  dim3 grid(args.num_tiles * args.base.nkv * args.head_blocks);
+  hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), grid, dim3(256), 0, stream, args);
+  return 0;
+}
 
 template <int HD, bool PAGE16>
 static int launch_prefill(const AttentionMfmaArgs& args, hipStream_t stream) {
@@ -110,12 +263,12 @@ extern "C" int ts_attention_prefill(const AttentionMfmaArgs* p, hipStream_t stre
   const AttentionArgs& a = args.base;
   if (a.num_tokens <= 0 || args.num_tiles <= 0) return 0;
   if (ts_check_attention_mfma_args(args, "attention_prefill")) return -1;
-  const bool page16 = a.page_size % 16 == 0;
+  const bool page16 = a.page_size >= 16 && (a.page_size & (a.page_size - 1)) == 0;
   int rc = 0;
   switch (a.hd) {
 #define TS_CASE(HD)                                                               \
   case HD:                                                                        \
-    rc = page16 ? launch_prefill<HD, true>(args, stream) : launch_prefill<HD, false>(args, stream); \
+    rc = page16 ? launch_prefill_lds<HD>(args, stream) : launch_prefill<HD, false>(args, stream); \
     break;
     TS_CASE(16) TS_CASE(32) TS_CASE(48) TS_CASE(64) TS_CASE(80) TS_CASE(96) TS_CASE(112)
     TS_CASE(128) TS_CASE(144) TS_CASE(160) TS_CASE(176) TS_CASE(192) TS_CASE(208) TS_CASE(224)

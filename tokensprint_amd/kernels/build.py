@@ -22,6 +22,9 @@ CSRC = Path(__file__).resolve().parent.parent / "csrc"
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # matrix-core results in ordinary vector registers: no copies to and from the
+         # accumulation registers around the float32 work between two products
+         "-mllvm", "-amdgpu-mfma-vgpr-form",
          "-Wno-unused-command-line-argument"]
 
 

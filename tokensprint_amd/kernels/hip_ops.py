@@ -389,7 +389,7 @@ class HipOps:
         # long portions of prompts: a wavefront takes several query tiles and walks alone
         tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
         if tiles16 * a.nkv * head_blocks >= 2048:
-            tpw = self.lib.ts_attention_prefill_tiles(a.hd)
+            tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size)
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
             m.num_splits = 1
