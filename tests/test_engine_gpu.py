@@ -108,3 +108,35 @@ def test_captured_decode_steps(setup):
             col.take(e, runner.step(e).clone())
             pos += 1
     drives.compare(col, {rid: ref[rid] for rid in ids}, rtol, atol)
+
+
+def test_captured_decode_steps_with_many_requests(setup):
+    """More than 16 requests decode together: the captured step then holds the vendor
+    library's matrix products; replayed several times with eager steps between."""
+    from tokensprint_amd.engine import StepEntry
+    model, page, requests, ref, (rtol, atol) = setup
+    runner = ModelRunner(model, page_size=page, num_pages=20 * (64 // page + 1), num_slots=20,
+                         graph_max_len=64)
+    toks = requests["r3"]                     # 40 tokens; 20 copies at staggered lengths
+    col = drives.Collector()
+    live = []
+    for i in range(20):
+        rc = runner.manager.admit(f"c{i}")
+        head = 10 + i
+        runner.manager.extend(rc, head)
+        runner.step([StepEntry(rc, toks[:head], 0, [])])
+        live.append([rc, head])
+    for step in range(6):
+        entries = []
+        for rc, pos in live:
+            runner.manager.extend(rc, pos + 1)
+            entries.append(StepEntry(rc, toks[pos:pos + 1], pos, [0]))
+        assert runner._graph_bucket(entries) == 20
+        logits = runner.step(entries).clone()
+        for (rc, pos), row in zip(live, logits):
+            torch.testing.assert_close(row.cpu(), ref["r3"][pos], rtol=rtol, atol=atol)
+        for item in live:
+            item[1] += 1
+        if step % 2 == 0:                     # eager work between replays
+            rc = live[0][0]
+            runner.step([StepEntry(rc, toks[:3], 0, [2])])

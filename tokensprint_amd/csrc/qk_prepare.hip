@@ -99,6 +99,91 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
   }
 }
 
+// The same for bfloat16 activations and head sizes 16, 32, 64, 128, 256: hd/8 lanes per
+// head, eight consecutive elements per lane in one 16-byte load, the rotation partner
+// (the element hd/2 further) fetched from the lane hd/16 further.  Values are written
+// transposed into their page, two bytes at a time.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_qk;
+typedef __attribute__((ext_vector_type(4))) float f32x4_qk;
+
+template <typename TC>
+__global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, int lanes_log2) {
+  const int L = 1 << lanes_log2;                     // lanes per head
+  const int heads_per_wave = kWave >> lanes_log2;
+  const int lane = threadIdx.x % kWave;
+  const int sub = lane & (L - 1);                    // my 8 elements: [8*sub, 8*sub + 8)
+  const int heads = a.nq + (a.store_kv ? 2 * a.nkv : 0);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t item = wave * heads_per_wave + (lane >> lanes_log2);
+  const bool live = item < (int64_t)a.num_tokens * heads;
+  const int64_t it = live ? item : 0;
+  const int t = (int)(it / heads), h = (int)(it % heads);
+  const int hd = a.hd, half = hd / 2;
+  const int pos = a.positions[t];
+  const int kind = h < a.nq ? 0 : (h < a.nq + a.nkv ? 1 : 2);
+  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * (a.nq + 2 * a.nkv) * hd + (int64_t)h * hd;
+  const bf16x8_qk x = *(const bf16x8_qk*)(src + sub * 8);
+  float v[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = (float)x[j];
+
+  const float* w = kind == 0 ? a.q_weight : a.k_weight;
+  if (kind != 2 && w) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+    for (int o = 1; o < L; o <<= 1) ss += __shfl_xor(ss, o, kWave);
+    const float rstd = rsqrtf(ss / (float)hd + a.eps);
+    const f32x4_qk w0 = *(const f32x4_qk*)(w + sub * 8), w1 = *(const f32x4_qk*)(w + sub * 8 + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[j] *= rstd * w0[j]; v[4 + j] *= rstd * w1[j]; }
+  }
+  if (kind != 2 && a.cos) {
+    const bool first = sub < L / 2;                  // holds elements i < hd/2
+    const int i0 = (sub & (L / 2 - 1)) * 8;          // index into the half-size table
+    const f32x4_qk c0 = *(const f32x4_qk*)(a.cos + (int64_t)pos * half + i0),
+                   c1 = *(const f32x4_qk*)(a.cos + (int64_t)pos * half + i0 + 4),
+                   s0 = *(const f32x4_qk*)(a.sin + (int64_t)pos * half + i0),
+                   s1 = *(const f32x4_qk*)(a.sin + (int64_t)pos * half + i0 + 4);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float other = __shfl_xor(v[j], L / 2, kWave);
+      const float c = j < 4 ? c0[j] : c1[j - 4], sn = j < 4 ? s0[j] : s1[j - 4];
+      // first half: re*c - im*s with im = other; second half: im*c + re*s with re = other
+      v[j] = first ? v[j] * c - other * sn : v[j] * c + other * sn;
+    }
+  }
+  if (!live) return;
+
+  if (kind == 0) {
+    bf16x8_qk o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = (bf16_t)v[j];
+    *(bf16x8_qk*)((bf16_t*)a.q_out + ((int64_t)t * a.nq + h) * hd + sub * 8) = o;
+    return;
+  }
+  const int kvh = kind == 1 ? h - a.nq : h - a.nq - a.nkv;
+  if (!a.paged) {
+    TC* dst = (TC*)(kind == 1 ? a.k_dst : a.v_dst) + ((int64_t)t * a.nkv + kvh) * hd + sub * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = from_f32<TC>(v[j]);
+    return;
+  }
+  const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
+  if (page < 0) return;
+  const int64_t head_base = ((int64_t)page * a.nkv + kvh) * a.page_size * hd;
+  const int slot = pos % a.page_size;
+  if (kind == 1) {
+    TC* dst = (TC*)a.k_dst + head_base + (int64_t)slot * hd + sub * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = from_f32<TC>(v[j]);
+  } else {
+    TC* dst = (TC*)a.v_dst + head_base + slot;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[(int64_t)(sub * 8 + j) * a.page_size] = from_f32<TC>(v[j]);
+  }
+}
+
 extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_type,
                              hipStream_t stream) {
   QkPrepareArgs a = *args;
@@ -113,6 +198,18 @@ extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_
   const int heads = a.nq + (a.store_kv ? 2 * a.nkv : 0);
   const int64_t items = (int64_t)a.num_tokens * heads;
   const int waves_per_block = 4;
+  if (act_type == TS_BF16 && a.hd >= 16 && a.hd <= 256 && (a.hd & (a.hd - 1)) == 0 &&
+      ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q_out & 15) == 0) {
+    const int lanes_log2 = __builtin_ctz(a.hd / 8);
+    const int heads_per_block = waves_per_block * (kWave >> lanes_log2);
+    const int64_t vblocks = (items + heads_per_block - 1) / heads_per_block;
+    if (vblocks > 2147483647LL) TS_FAIL("qk_prepare: too many tokens");
+    TS_DISPATCH_TYPE(cache_type, TC,
+        hipLaunchKernelGGL((qk_prepare_vec_kernel<TC>), dim3((unsigned)vblocks),
+                           dim3(waves_per_block * kWave), 0, stream, a, lanes_log2));
+    TS_CHECK_LAUNCH("qk_prepare");
+    return 0;
+  }
   const int64_t blocks = (items + waves_per_block - 1) / waves_per_block;
   if (blocks > 2147483647LL) TS_FAIL("qk_prepare: too many tokens");
   TS_DISPATCH_TYPE(act_type, T, TS_DISPATCH_TYPE(cache_type, TC,

@@ -166,8 +166,9 @@ class HipOps:
         N = weight.shape[0]
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
-        if self._library_ok(x, weight, out_dtype):
-            return torch.matmul(x, weight.t())
+        if self._library_ok(x, weight):
+            out = torch.matmul(x, weight.t())
+            return out if out_dtype == torch.bfloat16 else out.float()
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         if self._mfma_ok(x, weight):
             self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
@@ -180,13 +181,17 @@ class HipOps:
 
     # Rows from which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
     # torch.matmul), as the reference sends every linear layer to its vendor library
-    # (engine/nn/base_layers.py:7-10).  Below it the weight-streaming kernels are faster.
-    LIBRARY_ROWS = 192
+    # (engine/nn/base_layers.py:7-10).  Up to 16 rows (one matrix-core tile of A) the
+    # weight-streaming kernels here are faster and fuse the norm before and the SwiGLU
+    # after; measured inside captured graphs at the Qwen3-0.6B layer shapes, the library
+    # is ahead from 17 rows on.  Its result is bfloat16 (float32 accumulation), as the
+    # reference's logits are; float32 logits of more than 16 rows are that result widened.
+    LIBRARY_ROWS = 17
 
     @classmethod
-    def _library_ok(cls, x, weight, out_dtype):
+    def _library_ok(cls, x, weight, out_dtype=None):
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and out_dtype == torch.bfloat16 and x.shape[0] >= cls.LIBRARY_ROWS)
+                and x.shape[0] >= cls.LIBRARY_ROWS)
 
     @staticmethod
     def _mfma_ok(x, weight):
