@@ -140,18 +140,38 @@ def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
 @pytest.mark.parametrize("M,N,K", [(8, 4096, 1024), (1, 160, 96), (16, 112, 80), (3, 1024, 3072),
                                    (20, 96, 64), (5, 20000, 64)])
 def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
+    """Against float64.  In bfloat16 both the operand of the product (the normalised row)
+    and its results are rounded to 8 bits; which value exactly is rounded differs between
+    correct implementations (the fused kernel rounds x*w and divides by the root mean
+    square afterwards), so the bound is the rounding noise itself: a sum of K products of
+    operands with relative error 2^-9 has noise about 2^-9 * sqrt(K) * rms(x) * rms(w), a
+    rounded result 2^-9 of itself, and silu(g)*u inherits |u| times the noise of g plus
+    |silu(g)| times the noise of u."""
     resid = rand((M, K), torch.float32, gpu_device, 40)
     delta = rand((M, K), dtype, gpu_device, 41)
     nw = 1 + 0.1 * rand((K,), torch.float32, gpu_device, 42)
     w = rand((N, K), dtype, gpu_device, 43, scale=0.05)
     for d in (delta, None):
-        r_ref = resid.clone()
-        ref, r_ref = REF.norm_linear(r_ref, d, nw, 1e-5, w, dtype, silu_mul=silu)
+        x = resid.double() + (0 if d is None else d.double())
+        h = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
+        y = h @ w.double().T
+        # float32: sums in index order err by up to about sqrt(K) * 2^-24 per term magnitude
+        eps = 2.0 ** -9 if dtype == torch.bfloat16 else 2.0 ** -19
+        dot_noise = eps * (K ** 0.5) * float(h.pow(2).mean().sqrt() * w.double().pow(2).mean().sqrt())
+        noise = 4 * (dot_noise + eps * y.abs())
+        if silu:
+            g, u = y[:, :N // 2], y[:, N // 2:]
+            ref = torch.nn.functional.silu(g) * u
+            sg = torch.nn.functional.silu(g).abs()
+            bound = 1.2 * (u.abs() + noise[:, N // 2:]) * noise[:, :N // 2] + sg * noise[:, N // 2:] \
+                + 4 * eps * ref.abs()
+        else:
+            ref, bound = y, noise
         r_in = resid.clone()
         out, r_out = ops.norm_linear(r_in, d, nw, 1e-5, w, dtype, silu_mul=silu)
-        torch.testing.assert_close(r_out, r_ref, rtol=0, atol=0)
-        t = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
-        torch.testing.assert_close(out.float(), ref.float(), **t)
+        torch.testing.assert_close(r_out.double(), x, rtol=1e-6, atol=1e-6)
+        excess = ((out.double() - ref).abs() - bound).max()
+        assert excess <= 0, f"error exceeds the rounding bound by {float(excess):.3e}"
 
 
 def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):

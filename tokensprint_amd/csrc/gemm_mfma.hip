@@ -154,6 +154,7 @@ struct StagedArgs {
   int M, N, K;
   int delta_slabs, delta_is_f32;
   int kc;                   // K elements staged per round (multiple of WK*128, or >= K)
+  int rstd_offset;          // byte offset in LDS of the fused form's row factors
   float eps;
 };
 
@@ -167,6 +168,7 @@ __global__ __launch_bounds__(WN* WK* kWave) void gemm_staged_kernel(StagedArgs a
   const int xstride = a.kc + 8;                       // bf16 elements; 16 bytes of padding
   bf16_t* xs = (bf16_t*)smem;                         // [ROWS][xstride]
   f32x4* red = (f32x4*)smem;   // reuses the staging area once the K loop is over
+  float* rstd_s = (float*)(smem + a.rstd_offset);   // [rows], fused form only
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
   const int wn = wave % WN, wk = wave / WN;
   const int r = lane % 16, g = lane / 16;
@@ -199,10 +201,11 @@ __global__ __launch_bounds__(WN* WK* kWave) void gemm_staged_kernel(StagedArgs a
   };
 
   if (NORM) {
-    // Each wave takes rows m = wave, wave + NWAVES, ...: it sums the squares of a row,
-    // writes the new residual stream (workgroup column 0 only) and then stages the
-    // normalised row itself, so no barrier is needed between the two passes.  The
-    // fused form stages all of K at once (kc >= K).
+    // One pass: each wave takes rows m = wave, wave + NWAVES, ...; it writes the new
+    // residual stream (workgroup column 0 only), stages x * norm_w (not yet divided by
+    // the row's root mean square) and sums the squares.  The division commutes with the
+    // product, so it is applied to the accumulators at the end; nothing waits for the
+    // row sums.  The fused form stages all of K at once (kc >= K).
     for (int m = wave; m < rows; m += NWAVES) {
       float ss = 0.f;
       for (int u = lane; u < K / 8; u += kWave) {
@@ -213,22 +216,18 @@ __global__ __launch_bounds__(WN* WK* kWave) void gemm_staged_kernel(StagedArgs a
           *(f32x4*)op = f32x4{v[0], v[1], v[2], v[3]};
           *(f32x4*)(op + 4) = f32x4{v[4], v[5], v[6], v[7]};
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
-      }
-      const float rs = rsqrtf(wave_sum(ss) / (float)K + a.eps);
-      for (int u = lane; u < K / 8; u += kWave) {
-        float v[8];
-        stream8(m, u * 8, v);
         const f32x4 w0 = *(const f32x4*)(a.norm_w + u * 8), w1 = *(const f32x4*)(a.norm_w + u * 8 + 4);
         bf16x8 o;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          o[j] = (bf16_t)(v[j] * rs * w0[j]);
-          o[4 + j] = (bf16_t)(v[4 + j] * rs * w1[j]);
+          ss += v[j] * v[j] + v[4 + j] * v[4 + j];
+          o[j] = (bf16_t)(v[j] * w0[j]);
+          o[4 + j] = (bf16_t)(v[4 + j] * w1[j]);
         }
         *(bf16x8*)(xs + (size_t)m * xstride + u * 8) = o;
       }
+      ss = wave_sum(ss);
+      if (lane == 0) rstd_s[m] = rsqrtf(ss / (float)K + a.eps);
     }
   }
 
@@ -314,11 +313,14 @@ __global__ __launch_bounds__(WN* WK* kWave) void gemm_staged_kernel(StagedArgs a
   for (int mt = 0; mt < MT; ++mt) {
     const int m = m_base + mt * 16 + r;
     if (m >= M) continue;
+    const float rs = NORM ? rstd_s[mt * 16 + r] : 1.f;
     f32x4 v = acc[0][mt];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) v[t] *= rs;
     if (PAIR) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const float gt = (float)(bf16_t)acc[0][mt][t], up = (float)(bf16_t)acc[1][mt][t];
+        const float gt = (float)(bf16_t)v[t], up = (float)(bf16_t)(acc[1][mt][t] * rs);
         v[t] = gt / (1.f + expf(-gt)) * up;
       }
     }
@@ -340,7 +342,10 @@ static int launch_staged(StagedArgs a, hipStream_t stream) {
   const int staged_rows = NORM ? a.M : ROWS;
   const size_t lds_x = (size_t)staged_rows * (kc + 8) * 2;
   const size_t lds_red = (size_t)(WK - 1) * WN * NW * MT * kWave * 16;
-  const size_t lds = lds_x > lds_red ? lds_x : lds_red;
+  size_t lds = lds_x > lds_red ? lds_x : lds_red;
+  lds = (lds + 15) / 16 * 16;
+  a.rstd_offset = (int)lds;
+  if (NORM) lds += 64;      // up to 16 row factors
   if (lds > 150 * 1024) TS_FAIL("gemm_staged: %zu bytes of LDS needed", lds);
   auto kernel = gemm_staged_kernel<MT, WN, WK, TC, PAIR, NORM>;
   static bool raised = false;   // per instantiation
