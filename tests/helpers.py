@@ -31,7 +31,11 @@ TINY_C = qwen3_config(hidden=80, layers=4, heads=6, kv_heads=3, head_dim=48, int
                       vocab=301, eps=3e-6, theta=50000.0, tied=False, max_pos=512,
                       window=24, layer_types=["full_attention", "sliding_attention",
                                               "sliding_attention", "full_attention"])
-TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 8)}   # cfg, seed, page
+# head size 64: the smallest one the decode-fused kernels take
+TINY_D = qwen3_config(hidden=128, layers=2, heads=4, kv_heads=1, head_dim=64, inter=200,
+                      vocab=515, eps=2e-6, theta=2e5, tied=True, max_pos=320)
+TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 8),
+        "D": (TINY_D, 3, 32)}   # cfg, seed, page
 
 
 def random_prompt(length, vocab, seed):
