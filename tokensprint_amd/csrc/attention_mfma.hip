@@ -33,8 +33,10 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   const int kvh = (item / args.head_blocks) % a.nkv;
   const int hb = item % args.head_blocks;
   const int split = blockIdx.y;
-  const int entry = uniform(args.tiles[tile * 3]), tok0 = uniform(args.tiles[tile * 3 + 1]),
-            ntok = uniform(args.tiles[tile * 3 + 2]);
+  // without a tile list every entry brings one token (a decode step): tile = entry = token
+  const int entry = args.tiles ? uniform(args.tiles[tile * 3]) : tile,
+            tok0 = args.tiles ? uniform(args.tiles[tile * 3 + 1]) : tile,
+            ntok = args.tiles ? uniform(args.tiles[tile * 3 + 2]) : 1;
   const int* table = a.table + (int64_t)entry * a.table_width;
 
   // my query row: column r of S^T
@@ -154,7 +156,8 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
   const int tile = item / (a.nkv * args.head_blocks);
   const int kvh = (item / args.head_blocks) % a.nkv;
   const int hb = item % args.head_blocks;
-  const int tok0 = args.tiles[tile * 3 + 1], ntok = args.tiles[tile * 3 + 2];
+  const int tok0 = args.tiles ? args.tiles[tile * 3 + 1] : tile,
+            ntok = args.tiles ? args.tiles[tile * 3 + 2] : 1;
   const int group = a.nq / a.nkv;
   const int r = threadIdx.x / 16, dc = threadIdx.x % 16;
   const int ti = r / args.rows_per_token, hh = hb * 16 + r % args.rows_per_token;
@@ -166,6 +169,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
   const int nchunks = pos_last / kChunk - lo_tile / kChunk + 1;
   const int per = (nchunks - 1 + args.num_splits) / args.num_splits;
   const int used = min(args.num_splits, (nchunks + per - 1) / per);
+  // the loads of a split's statistics and of its values do not wait for one another
   float M = -INFINITY;
   for (int s = 0; s < used; ++s)
     M = fmaxf(M, args.partial_ml[(base + (int64_t)s * 16) * 2]);
@@ -174,11 +178,15 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
   for (int s = 0; s < used; ++s) {
     const int64_t slot = base + (int64_t)s * 16;
     const float ms = args.partial_ml[slot * 2];
-    if (ms == -INFINITY) continue;
-    const float w = __builtin_amdgcn_exp2f(ms - M);
-    L += args.partial_ml[slot * 2 + 1] * w;
+    const float ls = args.partial_ml[slot * 2 + 1];
+    float part[HD / 16];
 #pragma unroll
-    for (int i = 0; i < HD / 16; ++i) acc[i] += args.partial_o[slot * HD + i * 16 + dc] * w;
+    for (int i = 0; i < HD / 16; ++i) part[i] = args.partial_o[slot * HD + i * 16 + dc];
+    if (ms == -INFINITY) continue;       // an empty split wrote no values: ignore what is there
+    const float w = __builtin_amdgcn_exp2f(ms - M);
+    L += ls * w;
+#pragma unroll
+    for (int i = 0; i < HD / 16; ++i) acc[i] += part[i] * w;
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
   bf16_t* out = (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + kvh * group + hh) * HD;
@@ -218,7 +226,8 @@ int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who)
   if (args.rows_per_token != (group < 16 ? group : 16) ||
       args.head_blocks != (group + 15) / 16)
     TS_FAIL("%s: rows_per_token/head_blocks do not fit a group of %d", who, group);
-  if (!args.tiles) TS_FAIL("%s: no tile list", who);
+  if (!args.tiles && args.num_tiles != a.num_entries)
+    TS_FAIL("%s: without a tile list there is one tile per entry", who);
   if (((uintptr_t)a.q | (uintptr_t)a.out | (uintptr_t)a.k_pages | (uintptr_t)a.v_pages) & 15)
     TS_FAIL("%s: tensors must be 16-byte aligned", who);
   return 0;

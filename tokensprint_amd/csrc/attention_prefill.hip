@@ -263,6 +263,7 @@ extern "C" int ts_attention_prefill(const AttentionMfmaArgs* p, hipStream_t stre
   const AttentionArgs& a = args.base;
   if (a.num_tokens <= 0 || args.num_tiles <= 0) return 0;
   if (ts_check_attention_mfma_args(args, "attention_prefill")) return -1;
+  if (!args.tiles) TS_FAIL("attention_prefill: no tile list");
   const bool page16 = a.page_size >= 16 && (a.page_size & (a.page_size - 1)) == 0;
   int rc = 0;
   switch (a.hd) {

@@ -400,7 +400,10 @@ class HipOps:
             m.num_splits = 1
             self._call(self.lib.ts_attention_prefill, byref(m), self._stream())
             return
-        tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile)
+        if batch.max_q_len == 1:           # decode: tile i is entry i, no list needed
+            tiles_dev, num_tiles = None, batch.num_entries
+        else:
+            tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile)
         items = num_tiles * a.nkv * head_blocks
         chunk = self._attn_chunk
         span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
@@ -409,9 +412,10 @@ class HipOps:
         # few tiles (decode): a workgroup per tile and chunk, its waves share the chunk;
         # many tiles (prompts): a wavefront per tile walks its keys
         cooperative = items <= 1024
-        splits = min(max_chunks, max(1, (1024 if cooperative else 4096) // items))
+        splits = min(max_chunks, max(1, (512 if cooperative else 4096) // items))
         m.cooperative = int(cooperative)
-        m.tiles, m.num_tiles = tiles_dev.data_ptr(), num_tiles
+        m.tiles = tiles_dev.data_ptr() if tiles_dev is not None else None
+        m.num_tiles = num_tiles
         m.num_splits = splits
         if splits > 1:
             po = torch.empty(items * splits * 16 * a.hd, dtype=torch.float32, device=self.device)
