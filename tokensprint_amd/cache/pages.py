@@ -175,7 +175,21 @@ class CacheManager:
             out.append(max(0, total - len(table)) - released_now)
         return out
 
+    def _fits_as_is(self, rc: RequestCache, new_len: int) -> bool:
+        """True if no group has to take or give back a page for `new_len` tokens: the
+        common decode step, kept cheap."""
+        P = self.page_size
+        for g, table in enumerate(rc.tables):
+            if len(table) * P < new_len:
+                return False
+            if self.groups[g].window is not None and \
+                    self._first_kept_page(g, rc.num_tokens) > rc.released[g]:
+                return False
+        return True
+
     def can_extend(self, rc: RequestCache, new_len: int) -> bool:
+        if self._fits_as_is(rc, new_len):
+            return True
         return all(need <= pool.num_free
                    for need, pool in zip(self.pages_needed(rc, new_len), self.pools))
 
@@ -183,6 +197,9 @@ class CacheManager:
         """Make positions [rc.num_tokens, new_len) writable; all groups or none."""
         if new_len < rc.num_tokens:
             raise ValueError(f"cannot shrink a request from {rc.num_tokens} to {new_len}")
+        if self._fits_as_is(rc, new_len):
+            rc.num_tokens = new_len
+            return
         if not self.can_extend(rc, new_len):
             raise OutOfPages(
                 f"request {rc.request_id!r} needs {self.pages_needed(rc, new_len)} pages "

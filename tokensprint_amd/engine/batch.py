@@ -57,7 +57,7 @@ def _align(n: int, a: int = 4) -> int:
 def decode_layout(bucket: int, widths: list[int]):
     """Section offsets of a decode-only batch of `bucket` entries, one token each."""
     sizes = [bucket, bucket, bucket, bucket + 1, bucket, bucket, bucket] \
-        + [bucket * w for w in widths]
+        + [bucket * w for w in widths] + [bucket, 2 * bucket]     # ... temperatures, keys
     offs, total = [], 0
     for n in sizes:
         offs.append(total)
@@ -93,25 +93,54 @@ class StaticDecodeBatch:
         h[o[2]:o[2] + B] = np.arange(B)
         h[o[3]:o[3] + B + 1] = np.arange(B + 1)
         h[o[6]:o[6] + B] = np.arange(B)
+        for g, w in enumerate(widths):
+            h[o[7 + g]:o[7 + g] + B * w] = -1
+        # what each lane's block-table rows hold: (request cache, pages written) per group
+        self._lane = [[(None, 0)] * len(widths) for _ in range(B)]
+        G = len(widths)
+        # sampling inputs ride in the same buffer: float32 temperatures, int64 noise keys
+        self.temperatures = d[o[7 + G]:o[7 + G] + B].view(torch.float32)
+        self.keys = d[o[8 + G]:o[8 + G] + 2 * B].view(torch.int64)
+        self._h_temps = h[o[7 + G]:o[7 + G] + B].view(np.float32)
+        self._h_keys = h[o[8 + G]:o[8 + G] + 2 * B].view(np.int64)
 
-    def fill(self, entries) -> None:
+    def fill(self, entries, temperatures=None, keys=None) -> None:
         o, B, n = self.offs, self.bucket, len(entries)
         self.copied.synchronize()          # the last copy out of the pinned buffer is done
         h = self.host.numpy()
-        h[o[0]:o[0] + B] = 0
-        h[o[1]:o[1] + B] = 0
-        h[o[4]:o[4] + B] = 1
-        h[o[5]:o[5] + B] = 0
+        h[o[0] + n:o[0] + B] = 0
+        h[o[1] + n:o[1] + B] = 0
+        h[o[4] + n:o[4] + B] = 1
+        h[o[5] + n:o[5] + B] = 0
+        starts = [e.start for e in entries]
         h[o[0]:o[0] + n] = [e.tokens[0] for e in entries]
-        h[o[1]:o[1] + n] = [e.start for e in entries]
-        h[o[4]:o[4] + n] = [e.start + 1 for e in entries]
+        h[o[1]:o[1] + n] = starts
+        h[o[4]:o[4] + n] = np.asarray(starts, dtype=np.int32) + 1
         h[o[5]:o[5] + n] = [e.cache.slot for e in entries]
         for g, w in enumerate(self.widths):
-            tab = h[o[7 + g]:o[7 + g] + B * w].reshape(B, w)
-            tab[:] = -1
-            for i, e in enumerate(entries):
-                t = e.cache.tables[g]
-                tab[i, :len(t)] = t
+            base = o[7 + g]
+            for i in range(B):
+                rid, have = self._lane[i][g]
+                if i >= n:                               # idle lane: no pages
+                    if have or rid is not None:
+                        h[base + i * w:base + i * w + have] = -1
+                        self._lane[i][g] = (None, 0)
+                    continue
+                rc = entries[i].cache
+                t = rc.tables[g]
+                # same request as last step and nothing given back: only new pages to add
+                if rid is rc and have <= len(t) and rc.released[g] == 0:
+                    if have < len(t):
+                        h[base + i * w + have:base + i * w + len(t)] = t[have:]
+                else:
+                    h[base + i * w:base + i * w + max(have, len(t))] = -1
+                    h[base + i * w:base + i * w + len(t)] = t
+                self._lane[i][g] = (rc, len(t))
+        self._h_temps[:] = 0.0
+        self._h_keys[:] = 0
+        if temperatures is not None:
+            self._h_temps[:n] = temperatures
+            self._h_keys[:n] = keys
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 

@@ -104,8 +104,16 @@ class LLMEngine:
                 sampled_index.append(i)
             entries.append(StepEntry(req.cache, req.token_ids[lo:hi], lo,
                                      [req.num_new_tokens - 1] if last else []))
-        logits = self.runner.step(entries)
-        token_ids = self.sampler(logits, [reqs[i] for i in sampled_index])
+        token_ids = None
+        if len(sampled_index) == len(reqs):
+            # every entry ends in a draw: a decode step may run, draw included, as one graph
+            temps, keys = self.sampler.inputs(reqs)
+            drawn = self.runner.decode_and_sample(entries, temps, keys)
+            if drawn is not None:
+                token_ids = drawn.tolist()
+        if token_ids is None:
+            logits = self.runner.step(entries)
+            token_ids = self.sampler(logits, [reqs[i] for i in sampled_index])
         self.scheduler.postprocess(reqs, token_ids, sampled_index)
         outputs = [(r.ordinal, r.completion_token_ids) for r in reqs if r.is_finished]
         num_total_tokens = sum(len(r) for r in reqs if r.is_finished)

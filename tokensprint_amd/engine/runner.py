@@ -60,7 +60,7 @@ class ModelRunner:
         """Logits float32 [sum(len(e.want)), vocab], in the order of entries and want."""
         bucket = self._graph_bucket(entries)
         if bucket is not None:
-            return self._replay(bucket, entries)
+            return self._replay(bucket, entries)[0]
         return self.run(self.build(entries))
 
     # ------------------------------------------------------------ captured decode steps
@@ -90,11 +90,22 @@ class ModelRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.run(static.batch)
-        self.graphs[bucket] = (graph, static, logits)
+            # the draw is part of the captured step: rows with temperature 0 are greedy
+            tokens = self.model.ctx.ops.sample(logits, static.temperatures, static.keys)
+        self.graphs[bucket] = (graph, static, logits, tokens)
         return self.graphs[bucket]
 
-    def _replay(self, bucket: int, entries: list[StepEntry]) -> torch.Tensor:
-        graph, static, logits = self.graphs.get(bucket) or self._capture(bucket)
+    def decode_and_sample(self, entries: list[StepEntry], temperatures, keys):
+        """One decode step with the draw inside the captured graph: token ids (int32 device
+        tensor, one per entry), or None if the step does not fit a captured graph.
+        `temperatures` and `keys` are host sequences, one per entry."""
+        bucket = self._graph_bucket(entries)
+        if bucket is None:
+            return None
+        return self._replay(bucket, entries, temperatures, keys)[1][:len(entries)]
+
+    def _replay(self, bucket: int, entries: list[StepEntry], temperatures=None, keys=None):
+        graph, static, logits, tokens = self.graphs.get(bucket) or self._capture(bucket)
         vocab = self.model.spec.vocab_size
         for e in entries:
             if not 0 <= e.tokens[0] < vocab:
@@ -102,6 +113,6 @@ class ModelRunner:
             if e.start + 1 > e.cache.num_tokens:
                 raise ValueError(f"request {e.cache.request_id!r}: position {e.start} is not "
                                  "covered by its cache")
-        static.fill(entries)
+        static.fill(entries, temperatures, keys)
         graph.replay()
-        return logits[:len(entries)]
+        return logits[:len(entries)], tokens

@@ -40,6 +40,14 @@ class Sampler:
     def __init__(self, ops, device, engine_seed: int = 0) -> None:
         self.ops, self.device, self.engine_seed = ops, device, engine_seed
 
+    def inputs(self, requests):
+        """(temperatures, keys) as host lists, one per request: what the sampling kernel
+        takes.  A greedy request has temperature 0 and needs no key."""
+        temps = [r.temperature if r.temperature > 1e-10 else 0.0 for r in requests]
+        keys = [_signed(noise_key(self.engine_seed, r.seed, r.ordinal, r.num_completion_tokens))
+                if t > 0.0 else 0 for r, t in zip(requests, temps)]
+        return temps, keys
+
     def __call__(self, logits: torch.Tensor, requests) -> list[int]:
         """One token per row of logits; `requests[r]` has .temperature, .seed, .ordinal
         and .num_completion_tokens (the index of the token being drawn)."""
