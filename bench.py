@@ -119,6 +119,8 @@ def main() -> int:
     ap.add_argument("--model", default="qwen3-0.6b")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode run")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="only the 2,048-token prefill (for profiling); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -135,6 +137,12 @@ def main() -> int:
     item = 2 if dt_name == "bf16" else 4
     vocab = raw["vocab_size"]
 
+    if args.only_prefill:
+        model, pre_engine = make_engine(raw, args.dtype, layers, 1, ctx_len, 2048, page)
+        sec = prefill_run(pre_engine, 2048, vocab)
+        print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": 2048,
+                          "tok_per_s": round(2048 / sec, 1)}))
+        return 0
     model, engine = make_engine(raw, args.dtype, layers, args.batch, ctx_len, 2048, page)
     wbytes = weight_bytes(model)
     kv_per_token = 2 * layers * raw["num_key_value_heads"] * raw["head_dim"] * item
