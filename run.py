@@ -50,6 +50,8 @@ def parse_args(argv=None):
     ap.add_argument("--max-num-seqs", type=int, default=512)
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--chunked-prefill", type=_bool, default=False)
+    ap.add_argument("--prefix-caching", type=_bool, default=False,
+                    help="share cached full pages between requests with equal prefixes")
     ap.add_argument("--ignore-eos", type=_bool, default=False)
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args(argv)
@@ -91,7 +93,8 @@ def main(args) -> None:
         eos=eos, dtype=dtype, enforce_eager=args.enforce_eager,
         kvcache_block_size=args.page_size, num_kvcache_blocks=args.num_pages,
         max_num_batched_tokens=args.max_num_batched_tokens, max_num_seqs=args.max_num_seqs,
-        chunked_prefill=args.chunked_prefill, seed=args.seed)
+        chunked_prefill=args.chunked_prefill, seed=args.seed,
+        enable_prefix_caching=args.prefix_caching)
     engine = LLMEngine(model=model, config=config, tokenizer=tokenizer)
     params = SamplingParams(temperature=args.temperature, max_tokens=args.max_tokens,
                             ignore_eos=args.ignore_eos, seed=args.seed)

@@ -22,7 +22,7 @@ def paged_scenario(device, dtype, *, nkv, hd, page_size, spans, window=None, see
     manager = CacheManager(storage.groups, page_size, num_pages, len(spans))
     # scramble the free list
     order = torch.randperm(num_pages, generator=g).tolist()
-    manager.pools[0].free = type(manager.pools[0].free)(order)
+    manager.pools[0].free = type(manager.pools[0].free)((i, None) for i in order)
     entries = []
     # interleave allocation so that pages of different requests interleave too
     caches = [manager.admit(i) for i in range(len(spans))]
@@ -37,7 +37,7 @@ def paged_scenario(device, dtype, *, nkv, hd, page_size, spans, window=None, see
                 # do not let the window release pages while building the scenario
                 total = -(-target // page_size)
                 while len(rc.tables[0]) < total:
-                    rc.tables[0].append(manager.pools[0].take(rc.request_id))
+                    rc.tables[0].append(manager.pools[0].take())
                 rc.num_tokens = target
                 grown = True
     for rc, (s, n) in zip(caches, spans):

@@ -18,14 +18,19 @@ def manager(num_pages=8, page=4, windows=(None,), slots=4):
 
 def test_pool_fifo_and_double_free():
     pool = PagePool(3)
-    a, b = pool.take("x"), pool.take("x")
+    a, b = pool.take(), pool.take()
     assert (a, b) == (0, 1)                       # taken from the left
-    pool.give_back(a, "x")
+    pool.give_back(a)
     assert list(pool.free) == [2, 0]              # given back on the right
     with pytest.raises(RuntimeError, match="freed twice"):
-        pool.give_back(a, "x")
-    with pytest.raises(RuntimeError, match="owned by"):
-        pool.give_back(b, "y")
+        pool.give_back(a)
+    pool.take_tagged(b)                           # a second holder
+    pool.give_back(b)
+    assert pool.num_free == 2 and pool.refs[b] == 1
+    pool.give_back(b)
+    assert list(pool.free) == [2, 0, 1]
+    pool.take_tagged(0)                           # a particular free page, out of order
+    assert list(pool.free) == [2, 1] and pool.refs[0] == 1
     pool.check()
 
 
@@ -148,3 +153,111 @@ def test_random_orders_lose_nothing(seed):
     with pytest.raises(OutOfSlots):
         for i in range(4):
             m.admit(f"x{i}")
+
+
+# ------------------------------------------------------------------ prefix cache
+def test_prefix_cache_reuses_full_pages_but_never_the_last():
+    m = manager(num_pages=12, page=4)
+    m.enable_prefix_cache()
+    tokens = list(range(100, 118))                 # 18 tokens: pages 0..3 full, page 4 partial
+    a = m.admit("a", tokens)
+    assert a.num_tokens == 0                       # nothing cached yet
+    m.extend(a, 18)
+    m.register_full_pages(a, tokens, 18)
+    assert len(a.hashes) == 4 and len(m.prefix_index) == 4
+    # same prompt while "a" is live: its four full pages are shared
+    b = m.admit("b", tokens)
+    assert b.num_tokens == 16 and b.tables[0] == a.tables[0][:4]
+    assert [m.pools[0].refs[p] for p in b.tables[0]] == [2, 2, 2, 2]
+    m.extend(b, 18)
+    assert b.tables[0][4] != a.tables[0][4]        # the partial page is its own
+    m.check()
+    # a prompt of exactly 16 tokens may take only three pages: its last token is computed
+    c = m.admit("c", tokens[:16])
+    assert c.num_tokens == 12
+    m.free(c)
+    # another continuation shares only the common full pages
+    other = tokens[:8] + [7] * 10
+    d = m.admit("d", other)
+    assert d.num_tokens == 8 and d.tables[0] == a.tables[0][:2]
+    m.free(d); m.free(b); m.free(a)
+    assert m.pools[0].num_used == 0
+    # freed pages keep their contents until they are handed out for something else
+    e = m.admit("e", tokens)
+    assert e.num_tokens == 16
+    m.free(e)
+    m.check()
+
+
+def test_prefix_cache_forgets_evicted_pages_and_needs_full_groups():
+    m = manager(num_pages=4, page=4)
+    m.enable_prefix_cache()
+    tokens = list(range(12))
+    a = m.admit("a", tokens); m.extend(a, 12); m.register_full_pages(a, tokens, 12)
+    m.free(a)
+    b = m.admit("b", [50] * 16); m.extend(b, 16)   # takes all four pages: contents evicted
+    assert m.prefix_index == {}
+    m.free(b)
+    c = m.admit("c", tokens)
+    assert c.num_tokens == 0
+    m.free(c)
+    with pytest.raises(ValueError, match="keep all keys"):
+        manager(windows=(None, 8)).enable_prefix_cache()
+
+
+def test_chained_hash_depends_on_what_came_before():
+    h = CacheManager.block_hash
+    assert h([1, 2, 3, 4]) == h([1, 2, 3, 4])
+    assert h([1, 2, 3, 4]) != h([1, 2, 3, 5])
+    assert h([1, 2, 3, 4], h([9, 9, 9, 9])) != h([1, 2, 3, 4], h([8, 8, 8, 8]))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_orders_with_shared_prefixes(seed):
+    rnd = random.Random(seed)
+    m = manager(num_pages=rnd.choice([8, 14]), page=4, slots=3)
+    m.enable_prefix_cache()
+    stems = [[rnd.randrange(5) for _ in range(12)] for _ in range(2)]
+    live = {}
+    for step in range(300):
+        if rnd.random() < 0.3 and len(live) < 3:
+            tokens = rnd.choice(stems) + [rnd.randrange(5) for _ in range(rnd.randrange(1, 9))]
+            rc = m.admit(f"r{step}", tokens)
+            assert rc.num_tokens % 4 == 0 and rc.num_tokens < len(tokens)
+            live[f"r{step}"] = (rc, tokens)
+        elif rnd.random() < 0.7 and live:
+            rc, tokens = live[rnd.choice(sorted(live))]
+            n = min(len(tokens), rc.num_tokens + rnd.choice([1, 3, 8]))
+            if n > rc.num_tokens and m.can_extend(rc, n):
+                m.extend(rc, n)
+                m.register_full_pages(rc, tokens, n)
+        elif live:
+            rid = rnd.choice(sorted(live))
+            m.free(live.pop(rid)[0])
+        m.check()
+    for rc, _ in live.values():
+        m.free(rc)
+    m.check()
+    assert m.pools[0].num_used == 0
+
+
+def test_prefix_stops_at_the_first_miss_even_if_later_blocks_would_hit():
+    """The case of the reference's tests/test_block_manager.py:5-44: block 0 is a hit and in
+    use, block 1 has an index entry under its hash but other tokens, blocks 2 and 3 are
+    indexed and equal: one block is cached, three are new."""
+    P = 4
+    m = manager(num_pages=6, page=P)
+    m.enable_prefix_cache()
+    blocks = [[10] * P, [20] * P, [30] * P, [40] * P]
+    tokens = sum(blocks, [])
+    holder = m.admit("holder", tokens + [1]); m.extend(holder, 17)
+    m.register_full_pages(holder, tokens + [1], 17)
+    assert len(m.prefix_index) == 4
+    h1 = holder.hashes[1]
+    m.prefix_tokens[h1] = tuple([999] * P)         # same hash, other contents
+    hit = m.match_prefix(tokens + [2])
+    assert len(hit) == 1 and hit[0][1] == (holder.tables[0][0],)
+    rc = m.admit("new", tokens + [2])
+    assert rc.num_tokens == P                       # used: one block; new: the other three
+    m.free(rc); m.free(holder)
+    m.check()

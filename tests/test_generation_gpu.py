@@ -58,6 +58,33 @@ def test_greedy_is_the_same_however_the_work_is_cut(setup):
             assert engine.scheduler.num_preemptions > 0
 
 
+def test_prefix_cache_gives_the_same_tokens(setup):
+    """Prompts that share a stem of several pages, served one wave after another so that
+    later ones find the stem cached (live or already given back), under a pool small
+    enough that cached pages are also taken away again."""
+    cfg, d, model, page, prompts, expected = setup
+    if cfg.get("layer_types") and "sliding_attention" in cfg["layer_types"]:
+        with pytest.raises(ValueError, match="keep all keys"):
+            engine_for(model, d, torch.float32, kvcache_block_size=page,
+                       enable_prefix_caching=True)
+        return
+    pcfg, w = plain.read_model_dir(d)
+    stem = random_prompt(3 * page + 2, cfg["vocab_size"], 99)
+    tails = [random_prompt(n, cfg["vocab_size"], 200 + n) for n in (1, 4, page, 2 * page + 3)]
+    shared = [stem + t for t in tails] + [stem[:2 * page], stem]
+    want = [plain.greedy_generate(pcfg, w, p, 6) for p in shared]
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    for blocks in (64, -(-(len(shared[3]) + 8) // page) + 2):
+        engine = engine_for(model, d, torch.float32, kvcache_block_size=page,
+                            num_kvcache_blocks=blocks, enable_prefix_caching=True,
+                            max_num_seqs=2, max_model_len=cfg["max_position_embeddings"])
+        assert engine.generate(shared, sp, use_tqdm=False) == want, blocks
+        assert engine.generate(shared[::-1], sp, use_tqdm=False) == want[::-1], blocks
+        assert engine.scheduler.num_prefix_hit_tokens >= 3 * page
+        engine.runner.manager.check()
+        assert all(p.num_used == 0 for p in engine.runner.manager.pools)
+
+
 def test_first_tokens_and_a_one_token_prompt(setup):
     cfg, d, model, page, prompts, expected = setup
     engine = engine_for(model, d, torch.float32, kvcache_block_size=page, max_model_len=cfg["max_position_embeddings"])

@@ -209,3 +209,79 @@ def test_random_arrivals_with_a_tiny_pool_always_finish(seed):
         assert r.completion_token_ids == [(r.ordinal * 31 + n0 + i) % 50
                                           for i in range(r.max_tokens)]
     assert all(p.num_used == 0 for p in s.manager.pools)
+
+
+# ------------------------------------------------------------------ prefix cache
+def test_a_cached_prefix_is_not_computed_again():
+    s = make_scheduler(num_pages=12, budget=32, chunked=True)
+    s.manager.enable_prefix_cache()
+    stem = list(range(1, 11))                          # two full pages and a half
+    a = Request(0, stem + [40, 41], SamplingParams(max_tokens=2))
+    s.add_request(a)
+    assert s.schedule() == [a] and (a.num_cached_tokens, a.num_new_tokens) == (0, 12)
+    s.postprocess([a], [7], [0])
+    b = Request(1, stem + [50], SamplingParams(max_tokens=1))
+    s.add_request(b)
+    step = s.schedule()
+    assert step == [a, b]
+    assert (b.num_cached_tokens, b.num_new_tokens) == (8, 3)     # pages 0 and 1 shared
+    assert b.cache.tables[0][:2] == a.cache.tables[0][:2]
+    assert s.num_prefix_hit_tokens == 8
+    assert sum(r.num_new_tokens for r in step) == 4
+    s.postprocess(step, [8, 9], [0, 1])
+    assert a.is_finished and b.is_finished
+    assert s.manager.pools[0].num_used == 0
+    # finished requests leave their full pages findable: prompt and first completion token
+    c = Request(2, stem + [40, 41, 7, 8, 3], SamplingParams(max_tokens=1))
+    s.add_request(c)
+    s.schedule()
+    assert c.num_cached_tokens == 12
+    s.postprocess([c], [1], [0])
+    assert_queues(s)
+
+
+def test_a_prefix_hit_that_does_not_fit_leaves_nothing_behind():
+    s = make_scheduler(num_pages=5, budget=32, chunked=True)
+    s.manager.enable_prefix_cache()
+    a = Request(0, list(range(1, 13)), SamplingParams(max_tokens=8))
+    s.add_request(a)
+    s.postprocess(s.schedule(), [5], [0])              # 3 pages full, a fourth for the decode
+    s.postprocess(s.schedule(), [5], [0])
+    b = Request(1, list(range(1, 13)) + [9, 9, 9, 9, 9], SamplingParams(max_tokens=1))
+    s.add_request(b)                                   # shares 3 pages, needs 2 more: 1 free
+    assert s.schedule() == [a]
+    assert b.status == RequestStatus.WAITING and b.cache is None
+    assert s.num_prefix_hit_tokens == 0
+    assert [s.manager.pools[0].refs[p] for p in a.cache.tables[0]] == [1, 1, 1, 1]
+    assert_queues(s)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_arrivals_with_shared_prefixes_always_finish(seed):
+    rnd = random.Random(100 + seed)
+    s = make_scheduler(num_pages=rnd.choice([10, 14]), budget=rnd.choice([6, 16]),
+                       max_num_seqs=4, max_model_len=40, chunked=bool(seed % 2))
+    s.manager.enable_prefix_cache()
+    stems = [[rnd.randrange(50) for _ in range(9)] for _ in range(2)]
+    budget = s.max_num_batched_tokens
+    pending = [Request(i, (rnd.choice(stems) + [rnd.randrange(50) for _ in range(rnd.randrange(1, 8))])[:budget],
+                       SamplingParams(max_tokens=rnd.randrange(1, 12))) for i in range(12)]
+    everyone = list(pending)
+    steps = 0
+    while pending or not s.is_finished():
+        while pending and rnd.random() < 0.5:
+            s.add_request(pending.pop(0))
+        if s.is_finished():
+            continue
+        step = s.schedule()
+        sampled = [i for i, r in enumerate(step)
+                   if r.num_cached_tokens + r.num_new_tokens == len(r)]
+        tokens = [(step[i].ordinal * 31 + len(step[i])) % 50 for i in sampled]
+        s.postprocess(step, tokens, sampled)
+        assert_queues(s)
+        steps += 1
+        assert steps < 5000
+    for r in everyone:
+        assert r.is_finished and r.num_completion_tokens == r.max_tokens
+    assert s.num_prefix_hit_tokens > 0
+    assert all(p.num_used == 0 for p in s.manager.pools)

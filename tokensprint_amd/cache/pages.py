@@ -11,8 +11,11 @@ can see them; and fixed-size state slots, one per live request.
 
 from __future__ import annotations
 
-from collections import deque
+from collections import OrderedDict
 from dataclasses import dataclass, field
+
+import numpy as np
+import xxhash
 
 
 class OutOfPages(RuntimeError):
@@ -24,14 +27,21 @@ class OutOfSlots(RuntimeError):
 
 
 class PagePool:
-    """Fixed pool of page ids with a FIFO free list and an owner per page."""
+    """Fixed pool of page ids: a FIFO free list and a reference count per page.
+
+    A page is held by one request, or by several that share a cached prefix.  A free page
+    may still carry the hash of the block it held (`tag`), so that a later request with the
+    same prefix can take exactly that page back; the tag is dropped when the page is handed
+    out for something else (`on_evict` tells the prefix index)."""
 
     def __init__(self, num_pages: int) -> None:
         if num_pages < 1:
             raise ValueError(f"a pool needs at least one page, got {num_pages}")
         self.num_pages = num_pages
-        self.free: deque[int] = deque(range(num_pages))
-        self.owner: list[object | None] = [None] * num_pages   # None = free
+        self.free: OrderedDict[int, None] = OrderedDict((i, None) for i in range(num_pages))
+        self.refs: list[int] = [0] * num_pages
+        self.tag: list[int | None] = [None] * num_pages
+        self.on_evict = None               # callable(page, tag)
 
     @property
     def num_free(self) -> int:
@@ -41,35 +51,49 @@ class PagePool:
     def num_used(self) -> int:
         return self.num_pages - len(self.free)
 
-    def take(self, owner) -> int:
-        if owner is None:
-            raise ValueError("a page needs an owner")
+    def _evict_tag(self, page: int) -> None:
+        if self.tag[page] is not None:
+            if self.on_evict is not None:
+                self.on_evict(page, self.tag[page])
+            self.tag[page] = None
+
+    def take(self) -> int:
+        """The oldest free page, for new contents."""
         if not self.free:
             raise OutOfPages("no free page")
-        page = self.free.popleft()
-        if self.owner[page] is not None:
-            raise RuntimeError(f"page {page} is on the free list but owned by {self.owner[page]}")
-        self.owner[page] = owner
+        page, _ = self.free.popitem(last=False)
+        if self.refs[page] != 0:
+            raise RuntimeError(f"page {page} is on the free list with {self.refs[page]} holders")
+        self._evict_tag(page)
+        self.refs[page] = 1
         return page
 
-    def give_back(self, page: int, owner) -> None:
+    def take_tagged(self, page: int) -> None:
+        """Take a particular page for its contents: off the free list if nobody holds it,
+        one more holder otherwise."""
+        if self.refs[page] == 0:
+            if page not in self.free:
+                raise RuntimeError(f"page {page} has no holder and is not free")
+            del self.free[page]
+        self.refs[page] += 1
+
+    def give_back(self, page: int) -> None:
         if not 0 <= page < self.num_pages:
             raise RuntimeError(f"page id {page} out of range")
-        if self.owner[page] is None:
+        if self.refs[page] <= 0:
             raise RuntimeError(f"page {page} freed twice")
-        if self.owner[page] != owner:
-            raise RuntimeError(f"page {page} is owned by {self.owner[page]}, not {owner}")
-        self.owner[page] = None
-        self.free.append(page)
+        self.refs[page] -= 1
+        if self.refs[page] == 0:
+            self.free[page] = None         # to the right end: reused last, so a cached
+                                           # prefix survives as long as possible
 
     def check(self) -> None:
-        """No page lost, none held and free at once, none on the free list twice."""
-        free = list(self.free)
-        if len(set(free)) != len(free):
-            raise RuntimeError("a page is on the free list twice")
+        """No page lost, none held and free at once."""
         for page in range(self.num_pages):
-            if (self.owner[page] is None) != (page in set(free)):
-                raise RuntimeError(f"page {page}: free list and owner disagree")
+            if (self.refs[page] == 0) != (page in self.free):
+                raise RuntimeError(f"page {page}: free list and holder count disagree")
+            if self.refs[page] < 0:
+                raise RuntimeError(f"page {page}: negative holder count")
 
 
 class StateSlots:
@@ -127,6 +151,7 @@ class RequestCache:
     tables: list[list[int]]        # per group: logical page -> physical id, -1 = given back
     num_tokens: int = 0            # positions [0, num_tokens) are in the cache
     released: list[int] = field(default_factory=list)   # per group: leading pages given back
+    hashes: list[int] = field(default_factory=list)     # chained hash of every registered full page
 
 
 class CacheManager:
@@ -143,15 +168,94 @@ class CacheManager:
         self.pools = [PagePool(n) for n in counts]
         self.slots = StateSlots(num_slots)
         self.live: dict[object, RequestCache] = {}
+        # prefix cache (off until enabled): hash of a full page -> its page id in every group
+        self.prefix_index: dict[int, tuple[int, ...]] | None = None
+        self.prefix_tokens: dict[int, tuple[int, ...]] = {}   # the same keys: a page's tokens
+
+    # ------------------------------------------------------------ prefix cache
+    # The reference keeps a chained xxh64 per full block, a hash -> block map, blocks that
+    # keep their hash while free, reference counts for sharing, and never takes the last
+    # block of a request from the cache (engine/generation/block_manager.py:72-93,161-211,
+    # 406-475).  The same here, over all groups at once; only for models whose groups all
+    # keep every key (a window group gives pages back, so its prefix is not there to share).
+    def enable_prefix_cache(self) -> None:
+        if any(g.window is not None for g in self.groups):
+            raise ValueError("prefix caching needs every cache group to keep all keys")
+        if self.prefix_index is None:
+            self.prefix_index = {}
+            for g, pool in enumerate(self.pools):
+                pool.on_evict = lambda page, tag, g=g: self._evicted(g, page, tag)
+
+    def _evicted(self, g: int, page: int, tag: int) -> None:
+        entry = self.prefix_index.get(tag)
+        if entry is not None and entry[g] == page:
+            # one group's page is gone: the block is no longer whole
+            del self.prefix_index[tag]
+            self.prefix_tokens.pop(tag, None)
+            for g2, page2 in enumerate(entry):
+                if g2 != g and self.pools[g2].tag[page2] == tag:
+                    self.pools[g2].tag[page2] = None
+
+    @staticmethod
+    def block_hash(token_ids, prefix: int = -1) -> int:
+        """64-bit hash of a block of token ids chained to the hash of the blocks before."""
+        h = xxhash.xxh64()
+        if prefix != -1:
+            h.update(prefix.to_bytes(8, "little"))
+        h.update(np.asarray(token_ids, dtype=np.int64).tobytes())
+        return h.intdigest()
+
+    def match_prefix(self, token_ids) -> list[tuple[int, tuple[int, ...]]]:
+        """(hash, pages) of the leading full pages of `token_ids` that are cached, never
+        including the page that holds the last token."""
+        if self.prefix_index is None:
+            return []
+        P, out, h = self.page_size, [], -1
+        for i in range((len(token_ids) - 1) // P):
+            h = self.block_hash(token_ids[i * P:(i + 1) * P], h)
+            pages = self.prefix_index.get(h)
+            # a hit counts only with equal tokens (two blocks may share a hash), and the
+            # first miss ends the prefix whatever later blocks would match
+            if pages is None or self.prefix_tokens[h] != tuple(token_ids[i * P:(i + 1) * P]):
+                break
+            out.append((h, pages))
+        return out
+
+    def register_full_pages(self, rc: RequestCache, token_ids, computed: int) -> None:
+        """Make the pages of `rc` that are full and computed (positions < `computed`)
+        findable by their contents."""
+        if self.prefix_index is None:
+            return
+        P = self.page_size
+        full = min(computed, len(token_ids)) // P
+        while len(rc.hashes) < full:
+            i = len(rc.hashes)
+            h = self.block_hash(token_ids[i * P:(i + 1) * P], rc.hashes[-1] if rc.hashes else -1)
+            rc.hashes.append(h)
+            if h not in self.prefix_index:
+                pages = tuple(table[i] for table in rc.tables)
+                self.prefix_index[h] = pages
+                self.prefix_tokens[h] = tuple(token_ids[i * P:(i + 1) * P])
+                for g, page in enumerate(pages):
+                    self.pools[g].tag[page] = h
 
     # ------------------------------------------------------------ admission
-    def admit(self, request_id) -> RequestCache:
+    def admit(self, request_id, token_ids=None) -> RequestCache:
+        """A slot and empty block tables; with `token_ids` and the prefix cache enabled,
+        tables that already hold the request's cached prefix (rc.num_tokens tells how far)."""
         if request_id in self.live:
             raise RuntimeError(f"request {request_id!r} is already live")
         slot = self.slots.take(request_id)
         rc = RequestCache(request_id, slot, [[] for _ in self.groups],
                           released=[0] * len(self.groups))
         self.live[request_id] = rc
+        if token_ids is not None:
+            for h, pages in self.match_prefix(token_ids):
+                for g, page in enumerate(pages):
+                    self.pools[g].take_tagged(page)
+                    rc.tables[g].append(page)
+                rc.hashes.append(h)
+            rc.num_tokens = len(rc.hashes) * self.page_size
         return rc
 
     # ------------------------------------------------------------ growth
@@ -208,7 +312,7 @@ class CacheManager:
         total = -(-new_len // self.page_size)
         for g, table in enumerate(rc.tables):
             while len(table) < total:
-                table.append(self.pools[g].take(rc.request_id))
+                table.append(self.pools[g].take())
         rc.num_tokens = new_len
 
     def release_passed(self, rc: RequestCache) -> None:
@@ -217,7 +321,7 @@ class CacheManager:
             keep_from = min(self._first_kept_page(g, rc.num_tokens), len(table))
             for i in range(rc.released[g], keep_from):
                 if table[i] >= 0:
-                    self.pools[g].give_back(table[i], rc.request_id)
+                    self.pools[g].give_back(table[i])
                     table[i] = -1
             rc.released[g] = max(rc.released[g], keep_from)
 
@@ -230,30 +334,41 @@ class CacheManager:
         for g, table in enumerate(rc.tables):
             for page in reversed(table):
                 if page >= 0:
-                    self.pools[g].give_back(page, rc.request_id)
+                    self.pools[g].give_back(page)
             table.clear()
             rc.released[g] = 0
         self.slots.give_back(rc.slot, rc.request_id)
+        rc.hashes.clear()
         rc.num_tokens = 0
         del self.live[rc.request_id]
 
     # ------------------------------------------------------------ checks
     def check(self) -> None:
-        """Every used page is in exactly one live table; slots likewise."""
+        """Every page's holder count equals the live tables that name it; slots likewise."""
         for g, pool in enumerate(self.pools):
             pool.check()
-            seen: dict[int, object] = {}
+            holders = [0] * pool.num_pages
             for rc in self.live.values():
+                seen = set()
                 for page in rc.tables[g]:
                     if page < 0:
                         continue
                     if page in seen:
-                        raise RuntimeError(f"page {page} of group {g} is in two tables")
-                    seen[page] = rc.request_id
-                    if pool.owner[page] != rc.request_id:
-                        raise RuntimeError(f"page {page} of group {g}: owner mismatch")
-            if len(seen) != pool.num_used:
-                raise RuntimeError(f"group {g}: {pool.num_used} pages used, {len(seen)} in tables")
+                        raise RuntimeError(f"page {page} of group {g} twice in one table")
+                    seen.add(page)
+                    holders[page] += 1
+            if holders != pool.refs:
+                bad = next(i for i in range(pool.num_pages) if holders[i] != pool.refs[i])
+                raise RuntimeError(f"group {g} page {bad}: {pool.refs[bad]} holders counted, "
+                                   f"{holders[bad]} tables name it")
+            if self.prefix_index is None and max(holders, default=0) > 1:
+                raise RuntimeError(f"group {g}: a page is shared without a prefix cache")
+        if self.prefix_index is not None:
+            for h, pages in self.prefix_index.items():
+                for g, page in enumerate(pages):
+                    if self.pools[g].tag[page] != h:
+                        raise RuntimeError(f"prefix index names page {page} of group {g} "
+                                           "whose tag differs")
         slots = [rc.slot for rc in self.live.values()]
         if len(set(slots)) != len(slots):
             raise RuntimeError("a state slot is held twice")

@@ -46,6 +46,7 @@ class Config:
     chunked_prefill: bool = False
     dtype: torch.dtype = torch.bfloat16
     seed: int = 0
+    enable_prefix_caching: bool = False   # share cached full pages between equal prefixes
 
     def __post_init__(self) -> None:
         if not os.path.isdir(self.model):

@@ -38,6 +38,8 @@ class LLMEngine:
             model, page_size=page, num_pages=num_pages, num_slots=config.max_num_seqs,
             graph_max_len=None if config.enforce_eager or model.ctx.device.type != "cuda"
             else config.max_model_len)
+        if config.enable_prefix_caching:
+            self.runner.manager.enable_prefix_cache()
         self.scheduler = Scheduler(
             self.runner.manager, max_num_batched_tokens=config.max_num_batched_tokens,
             max_num_seqs=config.max_num_seqs, max_model_len=config.max_model_len,

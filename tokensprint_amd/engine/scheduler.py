@@ -42,6 +42,7 @@ class Scheduler:
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []
         self.num_preemptions = 0
+        self.num_prefix_hit_tokens = 0
 
     def is_finished(self) -> bool:
         return not self.waiting and not self.running
@@ -107,22 +108,25 @@ class Scheduler:
         if not preempted:
             while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
                 req = self.waiting[0]
-                n = len(req)
-                if self.enable_chunked:
-                    n = min(n, budget)
-                elif n > budget:
-                    # over budget: only a recomputed request, and only alone in its step
-                    if n <= self.max_num_batched_tokens or scheduled_running or scheduled_new:
-                        break
                 if self.manager.slots.num_free == 0:
                     break
-                rc = self.manager.admit(req.ordinal)
-                if not self.manager.can_extend(rc, n):
+                # with the prefix cache on, the request starts behind its cached pages
+                # (the reference's get_token_layout / allocate, scheduler.py:129-150)
+                rc = self.manager.admit(req.ordinal, req.token_ids)
+                cached = rc.num_tokens
+                n = len(req) - cached
+                if self.enable_chunked:
+                    n = min(n, budget)
+                # over budget: only a recomputed request, and only alone in its step
+                fits_budget = n <= budget or (n > self.max_num_batched_tokens
+                                              and not scheduled_running and not scheduled_new)
+                if not fits_budget or not self.manager.can_extend(rc, cached + n):
                     self.manager.free(rc)
                     break
-                self.manager.extend(rc, n)
+                self.num_prefix_hit_tokens += cached
+                self.manager.extend(rc, cached + n)
                 req.cache = rc
-                req.num_cached_tokens, req.num_new_tokens = 0, n
+                req.num_cached_tokens, req.num_new_tokens = cached, n
                 req.status = RequestStatus.RUNNING
                 self.waiting.popleft()
                 self.running.append(req)
@@ -155,6 +159,11 @@ class Scheduler:
         if len(token_ids) != len(sampled_index):
             raise ValueError("token_ids and sampled_index must have equal length, "
                              f"got {len(token_ids)} and {len(sampled_index)}.")
+        for req in reqs:
+            req.num_cached_tokens += req.num_new_tokens
+            req.num_new_tokens = 0
+            # before a finished request's pages go back: they stay findable while free
+            self.manager.register_full_pages(req.cache, req.token_ids, req.num_cached_tokens)
         for i, token in zip(sampled_index, token_ids):
             req = reqs[i]
             req.append_token(token)
@@ -169,7 +178,3 @@ class Scheduler:
                 req.cache = None
                 req.num_cached_tokens = req.num_new_tokens = 0
                 self.running.remove(req)
-        for req in reqs:
-            if req.status != RequestStatus.FINISHED:
-                req.num_cached_tokens += req.num_new_tokens
-                req.num_new_tokens = 0
