@@ -78,6 +78,13 @@ def test_silu_mul(ops, gpu_device, dtype):
                                **tol(dtype))
 
 
+def from_library(M, N, K):
+    """Whether a plain bfloat16 product of this shape goes to the vendor library: above 64
+    rows, and from 17 rows on where the kernels here lay their waves along N (a very wide
+    N or a short K)."""
+    return M > 64 or (M > 16 and (N >= 16384 or K < 512))
+
+
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("x_dtype,w_dtype", [(torch.float32, torch.float32),
                                              (torch.bfloat16, torch.bfloat16),
@@ -89,9 +96,8 @@ def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
     w = rand((N, K), w_dtype, gpu_device, 8, scale=0.1)
     out = ops.linear(x, w, out_dtype)
     ref = x.double() @ w.double().T
-    # bfloat16 operands with more than 16 rows go to the vendor library, whose result is
-    # bfloat16 also when float32 is asked for
-    widened = x_dtype == w_dtype == torch.bfloat16 and M > 16
+    # the vendor library's result is bfloat16 also when float32 is asked for
+    widened = x_dtype == w_dtype == torch.bfloat16 and from_library(M, N, K)
     t = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 and not widened \
         else dict(rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(out.double(), ref, **t)
@@ -100,26 +106,33 @@ def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (8, 1024, 3072),
                                    (17, 1000, 2048), (64, 6144, 1024), (3, 151936, 1024),
-                                   (130, 389, 96), (33, 50, 520), (70, 20000, 64)])
+                                   (130, 389, 96), (33, 50, 520), (70, 20000, 64),
+                                   (48, 1024, 3072), (64, 1024, 2048), (40, 3000, 1096),
+                                   (16, 300, 2056), (23, 520, 640)])
 def test_linear_bf16_matrix_core_shapes(ops, gpu_device, out_dtype, M, N, K):
     x = rand((M, K), torch.bfloat16, gpu_device, 17)
     w = rand((N, K), torch.bfloat16, gpu_device, 18, scale=0.05)
     out = ops.linear(x, w, out_dtype)
     ref = x.float() @ w.float().T
-    t = dict(rtol=2e-3, atol=2e-3) if out_dtype == torch.float32 and M <= 16 \
+    ours = not from_library(M, N, K)
+    t = dict(rtol=2e-3, atol=2e-3) if out_dtype == torch.float32 and ours \
         else dict(rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(out.float(), ref, **t)
-    # a row does not depend on the rest of the batch while our own kernels serve it (up
-    # to 16 rows); beyond that the vendor library does, and rows agree to rounding
+    # a row does not depend on the rest of the batch, bit for bit, while our own kernels
+    # serve it; beyond that the vendor library does, and rows agree to rounding
     one = ops.linear(x[M // 2:M // 2 + 1].contiguous(), w, out_dtype)
-    if M <= 16:
+    if ours:
         assert torch.equal(out[M // 2:M // 2 + 1], one)
+        last = ops.linear(x[M - 1:].contiguous(), w, out_dtype)
+        assert torch.equal(out[M - 1:], last)
     else:
         torch.testing.assert_close(out[M // 2:M // 2 + 1].float(), one.float(), rtol=1e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 160, 96), (40, 112, 80), (70, 1000, 520)])
+@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 160, 96), (40, 112, 80), (70, 1000, 520),
+                                   (40, 3072, 1024), (64, 1000, 2056), (33, 200, 520),
+                                   (5, 304, 3080)])
 def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
     x = rand((M, K), dtype, gpu_device, 19)
     w = rand((2 * I, K), dtype, gpu_device, 20, scale=0.1)
@@ -138,7 +151,8 @@ def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("silu", [False, True])
 @pytest.mark.parametrize("M,N,K", [(8, 4096, 1024), (1, 160, 96), (16, 112, 80), (3, 1024, 3072),
-                                   (20, 96, 64), (5, 20000, 64)])
+                                   (20, 96, 64), (5, 20000, 64), (16, 1000, 2056),
+                                   (9, 3072, 4096), (12, 520, 1096)])
 def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
     """Against float64.  In bfloat16 both the operand of the product (the normalised row)
     and its results are rounded to 8 bits; which value exactly is rounded differs between

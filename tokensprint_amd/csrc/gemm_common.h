@@ -1,0 +1,49 @@
+// What the matrix-core product kernels share: vector types, the K step of a wave, the
+// store of four results, and the one rule that lays the waves of a workgroup out.
+#pragma once
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kIterK = 128;   // K elements a wave consumes per iteration (4 MFMA steps)
+
+template <typename TC> __device__ __forceinline__ void store4(TC* p, f32x4 v, int n_left);
+template <> __device__ __forceinline__ void store4<float>(float* p, f32x4 v, int n_left) {
+  if (n_left >= 4 && ((uintptr_t)p & 15) == 0) { *(f32x4*)p = v; return; }
+  for (int t = 0; t < 4 && t < n_left; ++t) p[t] = v[t];
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v, int n_left) {
+  if (n_left >= 4 && ((uintptr_t)p & 7) == 0) {
+    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+    bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+    *(bf16x4*)p = o;
+    return;
+  }
+  for (int t = 0; t < 4 && t < n_left; ++t) p[t] = (bf16_t)v[t];
+}
+
+// How the waves of a workgroup are laid out: from N and K only, never from M, and the
+// same for every kernel, so that a row of C is computed in the same order whatever else
+// is in the batch and whichever kernel serves it.
+//   wide: 4 waves along N; deep: 8 waves split K; otherwise 4 waves split K.
+static inline bool layout_wide(int N, int K) { return N >= 16384 || K < 512; }
+static inline bool layout_deep(int K) { return K >= 2048; }
+
+// Operands of the product whose workgroups own 16 rows of W and split K among their
+// waves (every layout but the wide one).
+struct DirectArgs {
+  const bf16_t* A;          // [M, K], or null in the fused form
+  const bf16_t* W;          // [N, K] (pair: [2, N, K])
+  void* C;                  // [M, N]
+  const float* resid_in;    // fused form: [M, K]
+  const bf16_t* delta;      // fused form: [M, K] or null
+  const float* norm_w;      // fused form: [K]
+  float* resid_out;         // fused form: [M, K], written by workgroup column 0
+  int M, N, K;
+  float eps;
+};
+
+// Launches it; `norm` (the fused form) takes at most 16 rows.  Returns 0 or -1 with the
+// error text set.
+int gemm_direct_launch(const DirectArgs& a, int c_type, bool pair, bool norm, hipStream_t stream);

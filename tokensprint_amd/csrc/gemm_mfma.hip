@@ -11,27 +11,7 @@
 // sums in LDS in a fixed order (small N), so a result never depends on timing, and a
 // row of C does not depend on which other rows of A are in the call as long as the
 // launch shape is chosen from N and K alone.
-#include "common.h"
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-
-constexpr int kIterK = 128;   // K elements a wave consumes per iteration (4 MFMA steps)
-
-template <typename TC> __device__ __forceinline__ void store4(TC* p, f32x4 v, int n_left);
-template <> __device__ __forceinline__ void store4<float>(float* p, f32x4 v, int n_left) {
-  if (n_left >= 4 && ((uintptr_t)p & 15) == 0) { *(f32x4*)p = v; return; }
-  for (int t = 0; t < 4 && t < n_left; ++t) p[t] = v[t];
-}
-template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v, int n_left) {
-  if (n_left >= 4 && ((uintptr_t)p & 7) == 0) {
-    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-    bf16x4 o = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
-    *(bf16x4*)p = o;
-    return;
-  }
-  for (int t = 0; t < 4 && t < n_left; ++t) p[t] = (bf16_t)v[t];
-}
+#include "gemm_common.h"
 
 // MT: 16-row tiles of A per wave.  WN x WK = 4 waves: WN along N, WK along K.
 // PAIR: W holds two stacked matrices [2][N][K]; C = silu(A W0^T) * (A W1^T).
@@ -360,33 +340,14 @@ static int launch_staged(StagedArgs a, hipStream_t stream) {
   return 0;
 }
 
-static inline bool layout_wide(int N, int K);
-static inline bool layout_deep(int K);
-
+// Only the wide layout (4 waves along N) is served here; the layouts that split K among
+// the waves of a workgroup are gemm_direct.hip's.
 template <typename TC, bool PAIR, bool NORM>
 static int dispatch_staged(const StagedArgs& a, hipStream_t stream) {
-  const bool wide = layout_wide(a.N, a.K), deep = layout_deep(a.K);
-  if (NORM || a.M <= 16) {
-    if (wide) return launch_staged<1, 4, 1, TC, PAIR, NORM>(a, stream);
-    if (deep) return launch_staged<1, 1, 8, TC, PAIR, NORM>(a, stream);
-    return launch_staged<1, 1, 4, TC, PAIR, NORM>(a, stream);
-  }
-  if (a.M <= 32) {
-    if (wide) return launch_staged<2, 4, 1, TC, PAIR, false>(a, stream);
-    if (deep) return launch_staged<2, 1, 8, TC, PAIR, false>(a, stream);
-    return launch_staged<2, 1, 4, TC, PAIR, false>(a, stream);
-  }
-  if (wide) return launch_staged<4, 4, 1, TC, PAIR, false>(a, stream);
-  if (deep) return launch_staged<4, 1, 8, TC, PAIR, false>(a, stream);
-  return launch_staged<4, 1, 4, TC, PAIR, false>(a, stream);
+  if (NORM || a.M <= 16) return launch_staged<1, 4, 1, TC, PAIR, NORM>(a, stream);
+  if (a.M <= 32) return launch_staged<2, 4, 1, TC, PAIR, false>(a, stream);
+  return launch_staged<4, 4, 1, TC, PAIR, false>(a, stream);
 }
-
-// How the waves of a workgroup are laid out: from N and K only, never from M, and the
-// same for every kernel of this file, so that a row of C is computed in the same order
-// whatever else is in the batch and whichever kernel serves it.
-//   wide: 4 waves along N; deep: 8 waves split K; otherwise 4 waves split K.
-static inline bool layout_wide(int N, int K) { return N >= 16384 || K < 512; }
-static inline bool layout_deep(int K) { return K >= 2048; }
 
 template <int MT, int WN, int WK, typename TC, bool PAIR>
 static void launch_skinny(const bf16_t* A, const bf16_t* W, TC* C, int M, int N, int K,
@@ -402,9 +363,7 @@ static int dispatch_skinny(const void* a, const void* w, void* c, int M, int N, 
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
   if (M <= 16) {   // few rows: both operands straight from global memory
-    if (layout_wide(N, K)) launch_skinny<1, 4, 1, TC, PAIR>(A, W, (TC*)c, M, N, K, stream);
-    else if (layout_deep(K)) launch_skinny<1, 1, 8, TC, PAIR>(A, W, (TC*)c, M, N, K, stream);
-    else launch_skinny<1, 1, 4, TC, PAIR>(A, W, (TC*)c, M, N, K, stream);
+    launch_skinny<1, 4, 1, TC, PAIR>(A, W, (TC*)c, M, N, K, stream);
     return 0;
   }
   StagedArgs sa = {};
@@ -420,7 +379,11 @@ extern "C" int ts_gemm_mfma_bf16(const void* a, const void* w, void* c, int c_ty
   if (((uintptr_t)a | (uintptr_t)w) & 15) TS_FAIL("gemm_mfma: operands must be 16-byte aligned");
   if ((M + 63) / 64 > 65535) TS_FAIL("gemm_mfma: M=%d too large", M);
   int rc;
-  if (pair) {
+  if (!layout_wide(N, K)) {
+    DirectArgs da = {};
+    da.A = (const bf16_t*)a; da.W = (const bf16_t*)w; da.C = c; da.M = M; da.N = N; da.K = K;
+    rc = gemm_direct_launch(da, c_type, pair != 0, false, stream);
+  } else if (pair) {
     if (c_type != TS_BF16) TS_FAIL("gemm_mfma: the paired product writes bfloat16");
     rc = dispatch_skinny<bf16_t, true>(a, w, c, M, N, K, stream);
   } else if (c_type == TS_F32) {
@@ -435,6 +398,18 @@ extern "C" int ts_gemm_mfma_bf16(const void* a, const void* w, void* c, int c_ty
   return 0;
 }
 
+// Whether the fused form below takes a product of this shape: at most 16 rows, and in the
+// wide layout rows short enough for its staging buffer.
+extern "C" int ts_norm_gemm_mfma_fits(int M, int N, int K) {
+  if (M < 1 || M > 16 || K <= 0 || K % 8) return 0;
+  return !layout_wide(N, K) || (size_t)M * (K + 8) * 2 <= 140 * 1024;
+}
+
+// 0: 4 waves split K, 1: 8 waves split K, 2: wide (4 waves along N).
+extern "C" int ts_gemm_mfma_layout(int N, int K) {
+  return layout_wide(N, K) ? 2 : layout_deep(K) ? 1 : 0;
+}
+
 // Fused form for at most 16 rows: C = RMSNorm(resid_in + sum of delta slabs) W^T, and
 // resid_out = resid_in + sum of delta slabs.  delta may be null (slabs = 0).
 extern "C" int ts_norm_gemm_mfma_bf16(const float* resid_in, const void* delta, int delta_type,
@@ -442,14 +417,24 @@ extern "C" int ts_norm_gemm_mfma_bf16(const float* resid_in, const void* delta, 
                                       float* resid_out, const void* w, void* c, int c_type,
                                       int M, int N, int K, int pair, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 16) TS_FAIL("norm_gemm_mfma: at most 16 rows, got %d", M);
   if (K <= 0 || K % 8) TS_FAIL("norm_gemm_mfma: K=%d must be a positive multiple of 8", K);
-  if ((size_t)M * (K + 8) * 2 > 140 * 1024)
-    TS_FAIL("norm_gemm_mfma: %d rows of K=%d do not fit the staging buffer", M, K);
+  if (!ts_norm_gemm_mfma_fits(M, N, K))
+    TS_FAIL("norm_gemm_mfma: %d rows of K=%d are more than the fused form takes", M, K);
   if (((uintptr_t)w) & 15) TS_FAIL("norm_gemm_mfma: weights must be 16-byte aligned");
   if (!resid_in || !resid_out || resid_in == resid_out)
     TS_FAIL("norm_gemm_mfma: resid_in and resid_out must be two buffers");
   if (delta_slabs < 0 || (delta_slabs > 0 && !delta)) TS_FAIL("norm_gemm_mfma: delta slabs");
+  if (!layout_wide(N, K)) {
+    if (delta && (delta_slabs != 1 || delta_type != TS_BF16))
+      TS_FAIL("norm_gemm_mfma: this layout takes one bfloat16 delta");
+    DirectArgs da = {};
+    da.W = (const bf16_t*)w; da.C = c; da.M = M; da.N = N; da.K = K;
+    da.resid_in = resid_in; da.delta = (const bf16_t*)delta; da.norm_w = norm_w;
+    da.resid_out = resid_out; da.eps = eps;
+    if (gemm_direct_launch(da, c_type, pair != 0, true, stream)) return -1;
+    TS_CHECK_LAUNCH("norm_gemm_mfma");
+    return 0;
+  }
   StagedArgs sa = {};
   sa.W = (const bf16_t*)w; sa.C = c; sa.M = M; sa.N = N; sa.K = K;
   sa.resid_in = resid_in; sa.delta = delta; sa.norm_w = norm_w; sa.resid_out = resid_out;

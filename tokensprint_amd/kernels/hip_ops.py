@@ -179,19 +179,25 @@ class HipOps:
                        self._stream())
         return out
 
-    # Rows from which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
+    # Rows above which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
     # torch.matmul), as the reference sends every linear layer to its vendor library
-    # (engine/nn/base_layers.py:7-10).  Up to 16 rows (one matrix-core tile of A) the
-    # weight-streaming kernels here are faster and fuse the norm before and the SwiGLU
-    # after; measured inside captured graphs at the Qwen3-0.6B layer shapes, the library
-    # is ahead from 17 rows on.  Its result is bfloat16 (float32 accumulation), as the
-    # reference's logits are; float32 logits of more than 16 rows are that result widened.
-    LIBRARY_ROWS = 17
+    # (engine/nn/base_layers.py:7-10).  Up to 64 rows the weight-streaming kernels here
+    # are faster, measured inside captured graphs at the Qwen3-0.6B layer shapes, and fuse
+    # the norm before (up to 16 rows) and the SwiGLU after; in the wide layout (the output
+    # head) the library is ahead from 17 rows on.  Its result is bfloat16 (float32
+    # accumulation), as the reference's logits are; float32 results of such a product are
+    # that result widened.
+    LIBRARY_ROWS = 65
+    LIBRARY_ROWS_WIDE = 17
 
-    @classmethod
-    def _library_ok(cls, x, weight, out_dtype=None):
-        return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and x.shape[0] >= cls.LIBRARY_ROWS)
+    def _library_ok(self, x, weight, out_dtype=None):
+        if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            return False
+        M = x.shape[0]
+        if M >= self.LIBRARY_ROWS:
+            return True
+        return (M >= self.LIBRARY_ROWS_WIDE
+                and self.lib.ts_gemm_mfma_layout(weight.shape[0], weight.shape[1]) == 2)
 
     @staticmethod
     def _mfma_ok(x, weight):
@@ -211,8 +217,11 @@ class HipOps:
         self._check("weight", weight, self._FLOATS, ndim=2)
         if weight.shape[1] != K:
             raise ValueError(f"norm_linear: stream width {K}, weight has {weight.shape[1]} columns")
-        fused = (weight.dtype == torch.bfloat16 and M <= 16 and K % 8 == 0
-                 and M * (K + 8) * 2 <= 140 * 1024
+        N = weight.shape[0] // 2 if silu_mul else weight.shape[0]
+        fused = (weight.dtype == torch.bfloat16
+                 and self.lib.ts_norm_gemm_mfma_fits(M, N, K) == 1
+                 and (delta is None or delta.dtype == torch.bfloat16
+                      or self.lib.ts_gemm_mfma_layout(N, K) == 2)
                  and (out_dtype == torch.bfloat16 or not silu_mul)
                  and out_dtype in (torch.bfloat16, torch.float32))
         if not fused:
@@ -225,7 +234,6 @@ class HipOps:
         self._check("norm weight", norm_weight, torch.float32, shape=(K,))
         if delta is not None:
             self._check("delta", delta, self._FLOATS, shape=resid.shape)
-        N = weight.shape[0] // 2 if silu_mul else weight.shape[0]
         if silu_mul and weight.shape[0] % 2:
             raise ValueError("norm_linear: stacked gate/up weight needs an even row count")
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
