@@ -104,6 +104,16 @@ class TorchOps:
             self.kv_store(k.to(qkv.dtype), v, batch, table, cache)
         return q
 
+    def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
+               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window):
+        q = self.qk_norm_rope_store(
+            qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
+            num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight, k_weight=k_weight,
+            eps=eps, cos_sin=cos_sin)
+        return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
+                                    num_kv_heads=num_kv_heads, head_dim=head_dim,
+                                    scale=scale, window=window)
+
     # ---------------------------------------------------------------- attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
                         scale, window):

@@ -320,6 +320,98 @@ def test_paged_attention_long_portions(ops, gpu_device, nq, nkv, hd, page, windo
     torch.testing.assert_close(out[pick].float(), ref.float(), **tol(dtype))
 
 
+DECODE_SPANS = [(0, 1), (1, 1), (31, 1), (32, 1), (127, 1), (128, 1), (129, 1), (255, 1),
+                (256, 1), (700, 1), (1023, 1)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [None, 40, 300])
+@pytest.mark.parametrize("nq,nkv,hd,page", ATTN_SHAPES + [(16, 8, 128, 32), (8, 8, 64, 128),
+                                                          (6, 2, 160, 16), (20, 1, 32, 16)])
+def test_attend_in_a_decode_step(ops, gpu_device, dtype, nq, nkv, hd, page, window):
+    attend_decode_case(ops, gpu_device, dtype, nq, nkv, hd, page, window, DECODE_SPANS)
+
+
+@pytest.mark.parametrize("window", [None, 300])
+def test_attend_in_a_large_decode_step(ops, gpu_device, window):
+    """Enough entries that a tile's keys are not split over workgroups, and more than the
+    decode kernel takes at all."""
+    assert ops._decode_splits(8 * 3 * len(DECODE_SPANS), 1024) == 1
+    attend_decode_case(ops, gpu_device, torch.bfloat16, 16, 8, 128, 16, window, DECODE_SPANS * 3)
+    attend_decode_case(ops, gpu_device, torch.bfloat16, 16, 8, 128, 16, window, DECODE_SPANS * 7)
+
+
+def attend_decode_case(ops, gpu_device, dtype, nq, nkv, hd, page, window, spans):
+    """One new token per entry: norm, rotation, cache write and attention in one call (in
+    bfloat16 with a head size in steps of 32 and a power-of-two page: one kernel).  The
+    new key's slot holds garbage before the call, so a kernel that reads it instead of
+    using the step's own key shows."""
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=51)
+    T = batch.num_tokens
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 53)
+    wk = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 54)
+    angles = torch.outer(torch.arange(1100, dtype=torch.float32),
+                         1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    for b, (start, _) in enumerate(spans):               # poison the slots to be written
+        phys = int(table[b, start // page])
+        cache.k_pages[phys, :, start % page] = 1e4
+        cache.v_pages[phys, :, :, start % page] = -1e4
+    for kv_in_row, norm, rot in ((nkv, True, True), (nkv, False, True), (nkv, True, False),
+                                 (0, True, True)):
+        qkv = rand((T, (nq + 2 * kv_in_row) * hd), dtype, gpu_device, 52)
+        mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                           cache.k_pages.clone(), cache.v_pages.clone())
+        theirs = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                             cache.k_pages.clone(), cache.v_pages.clone())
+        if not kv_in_row:   # a run that reads another run's cache: the keys are there
+            for c in (mine, theirs):
+                c.k_pages.clamp_(-3, 3); c.v_pages.clamp_(-3, 3)
+        kw = dict(num_heads=nq, num_kv_heads=nkv, kv_in_row=kv_in_row, head_dim=hd,
+                  q_weight=wq if norm else None, k_weight=wk if norm else None, eps=1e-5,
+                  cos_sin=cos_sin if rot else None, scale=hd ** -0.5, window=window)
+        out = ops.attend(qkv, batch, table, mine, bool(kv_in_row), **kw)
+        ref = REF.attend(qkv, batch, table, theirs, bool(kv_in_row), **kw)
+        torch.testing.assert_close(mine.k_pages.float(), theirs.k_pages.float(), **tol(dtype))
+        torch.testing.assert_close(mine.v_pages.float(), theirs.v_pages.float(), rtol=0, atol=0)
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("window", [None, 1000])
+@pytest.mark.parametrize("fused", [True, False])
+def test_attend_decode_long_contexts_split_and_merge(ops, gpu_device, window, fused):
+    """Contexts long enough that a decode step's keys are split over workgroups and merged,
+    beside short ones whose later splits are empty."""
+    dtype = torch.bfloat16
+    nq, nkv, hd, page = 16, 8, 128, 16
+    spans = [(5000, 1), (2047, 1), (3, 1), (2049, 1)]
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=61)
+    assert ops._decode_splits(len(spans) * nkv, batch.max_ctx_len) > 3
+    T = batch.num_tokens
+    qkv = rand((T, (nq + 2 * nkv) * hd), dtype, gpu_device, 62)
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 63)
+    angles = torch.outer(torch.arange(5100, dtype=torch.float32),
+                         1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    theirs = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                         cache.k_pages.clone(), cache.v_pages.clone())
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, q_weight=wq, k_weight=wq, eps=1e-6,
+              cos_sin=cos_sin)
+    akw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
+    ref = REF.attend(qkv, batch, table, theirs, True, kv_in_row=nkv, **kw,
+                     scale=hd ** -0.5, window=window)
+    if fused:
+        out = ops.attend(qkv, batch, table, cache, True, kv_in_row=nkv, **kw,
+                         scale=hd ** -0.5, window=window)
+    else:
+        q = ops.qk_norm_rope_store(qkv, batch, table, cache, **kw)
+        out = ops.paged_attention(q, batch, table, cache, **akw)
+    torch.testing.assert_close(cache.k_pages.float(), theirs.k_pages.float(), **tol(dtype))
+    torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
     """One key among hundreds, at a page's edge, is made to dominate: the output must be

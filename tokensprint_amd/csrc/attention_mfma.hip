@@ -215,6 +215,20 @@ static int launch_mfma(const AttentionMfmaArgs& args, hipStream_t stream) {
   return 0;
 }
 
+// The merge alone, for the decode kernel's splits.
+int launch_attention_merge(const AttentionMfmaArgs& args, hipStream_t stream) {
+  const int items = args.num_tiles * args.base.nkv * args.head_blocks;
+  switch (args.base.hd) {
+#define TS_CASE(HD) case HD: hipLaunchKernelGGL(attention_merge_kernel<HD>, dim3(items), dim3(256), 0, stream, args); break;
+    TS_CASE(16) TS_CASE(32) TS_CASE(48) TS_CASE(64) TS_CASE(80) TS_CASE(96) TS_CASE(112)
+    TS_CASE(128) TS_CASE(144) TS_CASE(160) TS_CASE(176) TS_CASE(192) TS_CASE(208) TS_CASE(224)
+    TS_CASE(240) TS_CASE(256)
+#undef TS_CASE
+    default: TS_FAIL("attention_merge: head_dim=%d not built", args.base.hd);
+  }
+  return 0;
+}
+
 extern "C" int ts_attention_mfma_chunk() { return kChunk; }
 
 int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who) {

@@ -57,6 +57,14 @@ AttentionMfmaArgs._fields_ = [
 ]
 
 
+class AttentionDecodeArgs(Structure):
+    _fields_ = [
+        ("m", AttentionMfmaArgs), ("qkv", c_void_p), ("q_weight", c_void_p),
+        ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("eps", c_float),
+        ("kv_in_row", c_int),
+    ]
+
+
 def _load_library() -> ctypes.CDLL:
     path = find_library()
     if path is None:
@@ -384,11 +392,89 @@ class HipOps:
                                   head_dim, scale, window)
         if (q.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
                 and head_dim % 16 == 0 and head_dim <= 256 and cache.page_size % 4 == 0):
-            self._attention_mfma(a, batch, num_heads // num_kv_heads)
+            if self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads, head_dim,
+                                 cache.page_size, False):
+                self._attention_decode(a, batch, num_heads // num_kv_heads)
+            else:
+                self._attention_mfma(a, batch, num_heads // num_kv_heads)
         else:
             self._call(self.lib.ts_attention_generic, byref(a), _TYPE_CODE[q.dtype],
                        _TYPE_CODE[cache.k_pages.dtype], self._stream())
         return out
+
+    def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
+               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window):
+        """Everything between the q/k/v projection and the output projection: per-head
+        norm of q and k, rotation, the write of k and v into `cache` (if `write_cache`;
+        the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
+        over the cache -> [T, num_heads, head_dim].  A decode step (one token per entry)
+        in bfloat16 is one kernel; anything else is the preparation kernel and
+        paged_attention."""
+        T = qkv.shape[0]
+        fused = (qkv.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
+                 and bool(write_cache) == bool(kv_in_row)
+                 and self._decode_fits(batch, num_kv_heads, num_heads // num_kv_heads,
+                                       head_dim, cache.page_size, True))
+        if not fused:
+            q = self.qk_norm_rope_store(
+                qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
+                num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight,
+                k_weight=k_weight, eps=eps, cos_sin=cos_sin)
+            return self.paged_attention(q, batch, table, cache, num_heads=num_heads,
+                                        num_kv_heads=num_kv_heads, head_dim=head_dim,
+                                        scale=scale, window=window)
+        # the same argument checks as the preparation kernel's
+        qa = self._qk_args(qkv, batch, num_heads=num_heads, kv_in_row=kv_in_row,
+                           head_dim=head_dim, q_weight=q_weight, k_weight=k_weight, eps=eps,
+                           cos_sin=cos_sin)
+        self._check_cache(cache, table, batch, num_kv_heads, head_dim)
+        if T != batch.num_tokens or T != batch.num_entries:
+            raise ValueError("a decode step brings one token per entry")
+        out = torch.empty(T, num_heads, head_dim, dtype=qkv.dtype, device=self.device)
+        a = AttentionArgs()
+        self._fill_attention_args(a, None, out, batch, table, cache, num_heads, num_kv_heads,
+                                  head_dim, scale, window)
+        d = AttentionDecodeArgs()
+        d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
+        d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
+        self._attention_decode(a, batch, num_heads // num_kv_heads, d)
+        return out
+
+    def _attention_decode(self, a, batch, group, d=None):
+        """One token per entry: workgroups per (entry, key/value head, share of the keys)."""
+        d = d or AttentionDecodeArgs()
+        m = d.m
+        m.base = a
+        m.rows_per_token, m.head_blocks = min(group, 16), -(-group // 16)
+        m.num_tiles = batch.num_entries
+        items = m.num_tiles * a.nkv * m.head_blocks
+        span = batch.max_ctx_len if a.window == 0 else min(batch.max_ctx_len,
+                                                           a.window + self._attn_chunk)
+        m.num_splits = self._decode_splits(items, span)
+        if m.num_splits > 1:
+            po = torch.empty(items * m.num_splits * 16 * a.hd, dtype=torch.float32,
+                             device=self.device)
+            pml = torch.empty(items * m.num_splits * 16 * 2, dtype=torch.float32,
+                              device=self.device)
+            m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
+        self._call(self.lib.ts_attention_decode, byref(d), self._stream())
+
+    # Workgroups (entries x key/value heads) up to which a decode step takes the decode
+    # kernel; with more, the chip is full anyway and the smaller workgroups of the general
+    # kernel do better.  Measured in captured graphs at 16 query / 8 key heads of 128.
+    DECODE_ITEMS = 512
+
+    def _decode_fits(self, batch, num_kv_heads, group, head_dim, page_size, fused):
+        items = batch.num_entries * num_kv_heads * -(-group // 16)
+        return (batch.max_q_len == 1 and items <= self.DECODE_ITEMS
+                and self.lib.ts_attention_decode_fits(head_dim, page_size, int(fused)) == 1)
+
+    def _decode_splits(self, items, span):
+        """Workgroups per tile: enough to give every compute unit one or two, never more
+        than the context has 128-key chunks (a split without chunks costs an idle
+        workgroup and a line of the merge)."""
+        max_chunks = max(1, -(-span // self._attn_chunk))
+        return min(max_chunks, max(1, 192 // items))
 
     def _attention_mfma(self, a, batch, group):
         """Tile the batch's queries (16 rows of q heads x tokens per wavefront), choose how
@@ -448,8 +534,8 @@ class HipOps:
 
     def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
                              head_dim, scale, window):
-        T = q.shape[0]
-        a.q, a.out = q.data_ptr(), out.data_ptr()
+        T = out.shape[0]
+        a.q, a.out = (q.data_ptr() if q is not None else None), out.data_ptr()
         a.k_pages, a.v_pages = cache.k_pages.data_ptr(), cache.v_pages.data_ptr()
         a.positions, a.entry_of_token = batch.positions.data_ptr(), batch.entry_of_token.data_ptr()
         a.q_start, a.ctx_len = batch.q_start.data_ptr(), batch.ctx_len.data_ptr()

@@ -91,11 +91,11 @@ class GroupedQueryAttention(Mixer):
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None
         if fused:
-            q = ops.qk_norm_rope_store(
-                qkv, batch, table, cache if write_cache else None,
-                num_heads=self.nq, num_kv_heads=nkv_here, head_dim=self.hd,
+            o = ops.attend(
+                qkv, batch, table, cache, write_cache, num_heads=self.nq,
+                num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
-                cos_sin=tables)
+                cos_sin=tables, scale=self.scale, window=self.window)
         else:
             # the encoding has no rotary table: norm only, let it encode, then store
             q, k, v = ops.qk_norm_split(
@@ -104,7 +104,7 @@ class GroupedQueryAttention(Mixer):
             self.position.apply(q, k, batch.positions)
             if write_cache:
                 ops.kv_store(k, v, batch, table, cache)
-        o = ops.paged_attention(q, batch, table, cache, num_heads=self.nq,
-                                num_kv_heads=self.nkv, head_dim=self.hd,
-                                scale=self.scale, window=self.window)
+            o = ops.paged_attention(q, batch, table, cache, num_heads=self.nq,
+                                    num_kv_heads=self.nkv, head_dim=self.hd,
+                                    scale=self.scale, window=self.window)
         return ops.linear(o.view(T, self.nq * self.hd), self.w_o, self.ctx.dtype)
