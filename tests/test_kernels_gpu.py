@@ -199,15 +199,16 @@ def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,hd,page", [(4, 2, 16, 4), (8, 2, 32, 16), (6, 3, 48, 8),
                                             (16, 8, 128, 16), (5, 5, 80, 3), (8, 1, 256, 64)])
-def test_qk_norm_rope_store(ops, gpu_device, dtype, nq, nkv, hd, page):
-    spans = [(0, 9), (13, 1), (5, 20), (31, 2)]
+@pytest.mark.parametrize("spans", [[(0, 9), (13, 1), (5, 20), (31, 2)],
+                                   [(3, 70), (0, 33), (40, 1)]], ids=["short", "long"])
+def test_qk_norm_rope_store(ops, gpu_device, dtype, nq, nkv, hd, page, spans):
     batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
                                             spans=spans, seed=11)
     T = batch.num_tokens
     qkv = rand((T, (nq + 2 * nkv) * hd), dtype, gpu_device, 12)
     wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 13)
     wk = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 14)
-    angles = torch.outer(torch.arange(64, dtype=torch.float32),
+    angles = torch.outer(torch.arange(80, dtype=torch.float32),
                          1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
     cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
     ref_cache = type(cache)(cache.group, cache.page_size, cache.num_pages,

@@ -106,7 +106,12 @@ __global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfm
   const int group = a.nq / a.nkv;
   const int heads = a.nkv * args.head_blocks;
   const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
-  const int item = args.num_tiles - 1 - blockIdx.x / heads;    // longest key ranges first
+  // All workgroups of a prompt of a few thousand tokens are resident at once, two or
+  // three to a compute unit, in launch order: the first half of the launch takes the
+  // items with the longest key ranges, longest first, the second half the shortest,
+  // shortest first, so a unit's workgroups add up to about the same work.
+  const int rank = blockIdx.x / heads, half = (args.num_tiles + 1) / 2;
+  const int item = rank < half ? args.num_tiles - 1 - rank : rank - half;
   const int kvh = head_slot / args.head_blocks;
   const int hb = head_slot % args.head_blocks;
   const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
