@@ -1,16 +1,16 @@
 // C[M,N] = A[M,K] * W[N,K]^T for bfloat16 operands on the matrix cores, float32
-// accumulation, for the shapes where streaming W once is the whole cost: M from 1 to a
-// few hundred (decode batches, short portions of prompts, the output head).
+// accumulation, for the shapes where streaming W once is the whole cost: the entry
+// points of the matrix-core products, and the kernels of the wide layout (a very wide N,
+// the output head, or a short K), in which the four waves of a workgroup take different
+// tiles of 16 rows of W and nobody splits K.  The layouts that split K among a
+// workgroup's waves are gemm_direct.hip's.
 //
-// A wavefront owns a tile of 16 rows of W and up to 64 rows of A.  Both operands go from
-// global memory straight into the register layout of v_mfma_f32_16x16x32_bf16; every
-// lane reads 64 contiguous bytes of its row per iteration, so a row's four lanes cover
-// 256 contiguous bytes.  The K index that a register slot stands for is permuted the
-// same way for both operands, which a dot product does not notice.  Waves of a
-// workgroup either take different row tiles (large N) or split K and add their partial
-// sums in LDS in a fixed order (small N), so a result never depends on timing, and a
-// row of C does not depend on which other rows of A are in the call as long as the
-// launch shape is chosen from N and K alone.
+// Operands go from global memory into the register layout of v_mfma_f32_16x16x32_bf16;
+// every lane reads 64 contiguous bytes of its row per iteration, so a row's four lanes
+// cover 256 contiguous bytes.  The K index that a register slot stands for is permuted
+// the same way for both operands, which a dot product does not notice.  A result never
+// depends on timing, and a row of C does not depend on which other rows of A are in the
+// call as long as the launch shape is chosen from N and K alone.
 #include "gemm_common.h"
 
 // MT: 16-row tiles of A per wave.  WN x WK = 4 waves: WN along N, WK along K.
