@@ -155,7 +155,8 @@ def main() -> int:
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
 
     out = {
-        "metric": "decode tok/s at batch 8 (Qwen3-0.6B shape, 512-token prompts)",
+        "metric": f"decode tok/s at batch {args.batch} ({args.model} shape, "
+                  f"{args.prompt_len}-token prompts)",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dt_name,

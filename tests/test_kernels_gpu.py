@@ -152,7 +152,8 @@ def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
 @pytest.mark.parametrize("silu", [False, True])
 @pytest.mark.parametrize("M,N,K", [(8, 4096, 1024), (1, 160, 96), (16, 112, 80), (3, 1024, 3072),
                                    (20, 96, 64), (5, 20000, 64), (16, 1000, 2056),
-                                   (9, 3072, 4096), (12, 520, 1096)])
+                                   (9, 3072, 4096), (12, 520, 1096), (4, 1000, 2056),
+                                   (1, 3072, 4096), (3, 5000, 4096)])
 def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
     """Against float64.  In bfloat16 both the operand of the product (the normalised row)
     and its results are rounded to 8 bits; which value exactly is rounded differs between

@@ -281,7 +281,7 @@ static int tiles_per_workgroup(int M, int N, int most) {
 // four tiles 80), so that a wave's two or three steps of a decode product all are.
 template <typename TC, bool PAIR>
 static int dispatch(const DirectArgs& a, bool norm, hipStream_t stream) {
-  const bool deep = layout_deep(a.K);
+  const bool deep = layout_deep(a.N, a.K);
   if (norm) {
     if (deep) launch<1, 8, TC, PAIR, true, 2, 3>(a, stream);
     else launch<1, 4, TC, PAIR, true, 4, 2>(a, stream);

@@ -398,16 +398,19 @@ extern "C" int ts_gemm_mfma_bf16(const void* a, const void* w, void* c, int c_ty
   return 0;
 }
 
-// Whether the fused form below takes a product of this shape: at most 16 rows, and in the
-// wide layout rows short enough for its staging buffer.
+// Whether the fused form below takes a product of this shape: at most 16 rows; in the
+// wide layout rows short enough for its staging buffer; in the others at most 16384
+// elements of the residual stream (16 rows of 1024, 4 of 4096), because every workgroup
+// reads them in float32 and with a long K that costs more than the norm kernel saved.
 extern "C" int ts_norm_gemm_mfma_fits(int M, int N, int K) {
   if (M < 1 || M > 16 || K <= 0 || K % 8) return 0;
-  return !layout_wide(N, K) || (size_t)M * (K + 8) * 2 <= 140 * 1024;
+  if (layout_wide(N, K)) return (size_t)M * (K + 8) * 2 <= 140 * 1024;
+  return (int64_t)M * K <= 16384;
 }
 
 // 0: 4 waves split K, 1: 8 waves split K, 2: wide (4 waves along N).
 extern "C" int ts_gemm_mfma_layout(int N, int K) {
-  return layout_wide(N, K) ? 2 : layout_deep(K) ? 1 : 0;
+  return layout_wide(N, K) ? 2 : layout_deep(N, K) ? 1 : 0;
 }
 
 // Fused form for at most 16 rows: C = RMSNorm(resid_in + sum of delta slabs) W^T, and
