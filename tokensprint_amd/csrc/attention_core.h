@@ -6,6 +6,7 @@
 //   Q operand   lane (r, g) holds Q[row r][g*8*KS + s*8 + j]                 (B)
 //   S^T result  lane (r, g) holds S^T[key blk*16 + g*4 + t][row r]
 //   V operand   lane (r, g) holds V^T[d = db*16 + r][keys blk0: g*4..+3, blk1: g*4..+3]
+//               (one 8-element register group per 16 head elements)
 //   P operand   lane (r, g) holds its own 8 probabilities, in that key order
 // so a lane's scores are, in place, its part of the second product's B operand, and the
 // softmax statistics of a query row live in the four lanes r, r+16, r+32, r+48.
@@ -23,7 +24,7 @@ struct KvBlock {
   static constexpr int KS = (HD + 31) / 32;
   static constexpr int DB = HD / 16;
   bf16x8 k[2][KS];
-  bf16x4 v[2][DB];
+  bf16x8 v[DB];        // [0..3]: keys of the first 16-key block, [4..7]: of the second
 };
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
@@ -80,6 +81,7 @@ __device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArg
   const int last_key = cur.last_key;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const bf16x4 zero4 = {0, 0, 0, 0};
+  bf16x4 vh[2][DB];
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
     const int k0 = kb + blk * 16;                        // first key of the 16-key block
@@ -96,12 +98,12 @@ __device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArg
         }
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          b.v[blk][db] = *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P);
+          vh[blk][db] = *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P);
       } else {
 #pragma unroll
         for (int s = 0; s < KS; ++s) b.k[blk][s] = zero8;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) b.v[blk][db] = zero4;
+        for (int db = 0; db < DB; ++db) vh[blk][db] = zero4;
       }
     } else {
       const int key = k0 + r;
@@ -117,9 +119,12 @@ __device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArg
       const bf16_t* vcol = vp + ((int64_t)max(vpage, 0) * a.nkv + kvh) * HD * P + key4 % P;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        b.v[blk][db] = vpage >= 0 ? *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P) : zero4;
+        vh[blk][db] = vpage >= 0 ? *(const bf16x4*)(vcol + (int64_t)(db * 16 + r) * P) : zero4;
     }
   }
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+    b.v[db] = __builtin_shufflevector(vh[0][db], vh[1][db], 0, 1, 2, 3, 4, 5, 6, 7);
   if (PAGE16) cur.start(kb + stride);
 }
 
@@ -151,8 +156,11 @@ __device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow,
 }
 
 // Scores of the block for one tile, masked softmax update, and O^T += V^T P^T.
-// `interior`: every key of the block is visible to every row of the tile (wave-uniform),
-// so the mask is skipped.  scale_log2 = softmax scale * log2(e); m is kept in that unit.
+// `interior` (wave-uniform): every key of the block is visible to every row of the tile,
+// so the mask is skipped: by a branch around it, the rest is one stretch of code either
+// way.  scale_log2 = softmax scale * log2(e); m is kept in that unit.  A row that has
+// seen no key yet has m = -inf; the exponentials take a finite stand-in for it, which
+// makes all of them 0 without a special case.
 template <int HD>
 __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>& b, int kb,
                                             float scale_log2, bool interior, int g) {
@@ -165,29 +173,27 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
     for (int s = 0; s < KS; ++s)
       st[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.k[blk][s], t.q[s], st[blk], 0, 0, 0);
   }
-  float sv[8];
-  float mx = -INFINITY;
+  if (!interior) {
+    asm volatile("" ::: "memory");   // keeps this a branch: blended in, it costs every block
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk)
+    for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float s = st[blk][i] * scale_log2;
-      if (!interior) {
+      for (int i = 0; i < 4; ++i) {
         const int key = kb + blk * 16 + g * 4 + i;
-        s = (key <= t.pos && key >= t.lo) ? s : -INFINITY;
+        st[blk][i] = (key <= t.pos && key >= t.lo) ? st[blk][i] : -INFINITY;
       }
-      sv[blk * 4 + i] = s;
-      mx = fmaxf(mx, s);
-    }
-  mx = col4_max(mx);
-  const float m_new = fmaxf(t.m, mx);
-  const bool any = m_new != -INFINITY;
-  const float corr = any ? __builtin_amdgcn_exp2f(t.m - m_new) : 1.f;
+  }
+  float mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
+                   fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+  // the scale is positive: the largest score stays the largest
+  const float m_new = fmaxf(t.m, col4_max(mx) * scale_log2);
+  const float m_use = fmaxf(m_new, -1e30f);
+  const float corr = __builtin_amdgcn_exp2f(t.m - m_use);
   float ps = 0.f;
   bf16x8 pv;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float p = any ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.f;
+    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i / 4][i % 4], scale_log2, -m_use));
     ps += p;
     pv[i] = (bf16_t)p;
   }
@@ -196,12 +202,10 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
   t.m = m_new;
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
-    const bf16x4 v0 = b.v[0][db], v1 = b.v[1][db];
-    const bf16x8 vfull = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
     f32x4 acc = t.o[db];
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] *= corr;
-    t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfull, pv, acc, 0, 0, 0);
+    t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[db], pv, acc, 0, 0, 0);
   }
 }
 

@@ -90,16 +90,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
 // (page sizes that are powers of two from 16 up).  The waves take four consecutive query tiles of
 // one entry and one key/value head; per block of 32 keys each wave fetches a quarter of
 // the operand registers from global memory and stores them to LDS in operand layout,
-// double-buffered: the fetch of block i+1 is in flight while block i is worked on, and
-// one barrier per block separates the two.  A block is read from L2 once per workgroup
+// double-buffered: the fetch of the next block is in flight while a block is worked on,
+// and one barrier per block separates the two.  A block is read from L2 once per workgroup
 // instead of once per wave, and operands come out of LDS just before their product, so
 // few registers are held and several workgroups share a CU.
 template <int HD>
-__global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfmaArgs args) {
+__global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_kernel(
+    AttentionMfmaArgs args) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
   constexpr int KQ = (2 * KS + 3) / 4, VQ = (2 * DB + 3) / 4;    // operand slots per wave
   __shared__ bf16x8 k_lds[2][2 * KS][kWave];
-  __shared__ bf16x4 v_lds[2][2 * DB][kWave];
+  __shared__ bf16x8 v_lds[2][DB][kWave];     // low half: first 16-key block, high: second
   const AttentionArgs& a = args.base;
   const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int r = lane % 16, g = lane / 16;
@@ -152,9 +153,17 @@ __global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfm
   // issued unconditionally (a missing page reads page 0 and is zeroed when stored to
   // LDS), so nothing but the barrier stands between them and the work on the block.
   constexpr bool kEven = (2 * KS) % 4 == 0, vEven = (2 * DB) % 4 == 0;
-  bf16x8 kreg[KQ];
-  bf16x4 vreg[VQ];
-  bool kvalid[KQ], vvalid[VQ];                  // wave-uniform
+  // kAhead blocks are on their way from memory while one is worked on.  More than one
+  // was measured and does not pay: the registers they take cost a resident wave, and it
+  // is the number of resident waves (four per SIMD up to head size 128) that hides the
+  // waits of this kernel, those for memory among them.
+  constexpr int kAhead = 1;
+  struct Fetched {
+    bf16x8 k[KQ];
+    bf16x4 v[VQ];
+    bool kvalid[KQ], vvalid[VQ];                // wave-uniform
+  };
+  Fetched ring[kAhead];
   // address = head base + page * page stride (scalar) + position in page (scalar)
   //           + this lane's offset inside the slot (fixed for the whole walk)
   const int64_t k_page_stride = (int64_t)a.nkv * P * HD, v_page_stride = k_page_stride;
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfm
     v_blk[i] = q / DB;
     v_lane[i] = ((q % DB) * 16 + r) * P + g * 4;
   }
-  auto fetch = [&](int kb) {
+  auto fetch = [&](Fetched& f, int kb) {
     const int in_page = kb & (P - 1);             // a block of 16 keys never straddles a page
     const int page0 = cur.next0, page1 = cur.next1;
     const bf16_t* kb0 = k_head + (int64_t)max(page0, 0) * k_page_stride + in_page * HD;
@@ -186,47 +195,56 @@ __global__ __launch_bounds__(256) void attention_prefill_lds_kernel(AttentionMfm
     const bf16_t* vb1 = v_head + (int64_t)max(page1, 0) * v_page_stride + ((in_page + 16) & (P - 1));
 #pragma unroll
     for (int i = 0; i < KQ; ++i) {
-      kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
-      kreg[i] = *(const bf16x8*)((k_blk[i] ? kb1 : kb0) + k_lane[i]);
+      f.kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
+      f.k[i] = *(const bf16x8*)((k_blk[i] ? kb1 : kb0) + k_lane[i]);
     }
 #pragma unroll
     for (int i = 0; i < VQ; ++i) {
-      vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
-      vreg[i] = *(const bf16x4*)((v_blk[i] ? vb1 : vb0) + v_lane[i]);
+      f.vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
+      f.v[i] = *(const bf16x4*)((v_blk[i] ? vb1 : vb0) + v_lane[i]);
     }
     cur.start(kb + 32);
   };
-  auto stash = [&](int buf) {                      // registers -> LDS, operand layout
+  auto stash = [&](const Fetched& f, int buf) {    // registers -> LDS, operand layout
 #pragma unroll
     for (int i = 0; i < KQ; ++i)
       if (kEven || wave + 4 * i < 2 * KS)
-        k_lds[buf][wave + 4 * i][lane] = kvalid[i] ? kreg[i] : zero8;
+        k_lds[buf][wave + 4 * i][lane] = f.kvalid[i] ? f.k[i] : zero8;
 #pragma unroll
     for (int i = 0; i < VQ; ++i)
       if (vEven || wave + 4 * i < 2 * DB)
-        v_lds[buf][wave + 4 * i][lane] = vvalid[i] ? vreg[i] : zero4;
+        ((bf16x4*)&v_lds[buf][(wave + 4 * i) % DB][lane])[(wave + 4 * i) / DB] =
+            f.vvalid[i] ? f.v[i] : zero4;
   };
 
-  fetch(key_begin);
-  stash(0);
+#pragma unroll
+  for (int p = 0; p < kAhead; ++p)
+    if (key_begin + 32 * p <= pos_last) fetch(ring[p], key_begin + 32 * p);
+  stash(ring[0], 0);
   __syncthreads();
   int buf = 0;
-  for (int kb = key_begin; kb <= pos_last; kb += 32, buf ^= 1) {
-    const bool more = kb + 32 <= pos_last;
-    if (more) fetch(kb + 32);
-    if (kb <= tile_last && kb + 31 >= tile_lo) {
-      KvBlock<HD> b;
+  // ring slot p holds block kb0 + 32 p, already in LDS when its turn comes, and is
+  // fetched into again at once for the block kAhead further on
+  for (int kb0 = key_begin; kb0 <= pos_last; kb0 += 32 * kAhead) {
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
+    for (int p = 0; p < kAhead; ++p) {
+      const int kb = kb0 + 32 * p;
+      if (kb > pos_last) break;
+      if (kb + 32 * kAhead <= pos_last) fetch(ring[p], kb + 32 * kAhead);
+      if (kb <= tile_last && kb + 31 >= tile_lo) {
+        KvBlock<HD> b;
 #pragma unroll
-        for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = k_lds[buf][blk * KS + s0][lane];
+        for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int db = 0; db < DB; ++db) b.v[blk][db] = v_lds[buf][blk * DB + db][lane];
+          for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = k_lds[buf][blk * KS + s0][lane];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) b.v[db] = v_lds[buf][db][lane];
+        tile_update<HD>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
       }
-      tile_update<HD>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
+      if (kb + 32 <= pos_last) stash(ring[(p + 1) % kAhead], buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
     }
-    if (more) stash(buf ^ 1);
-    __syncthreads();
   }
   if (row_ok)
     store_tile<HD>(t, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
