@@ -26,9 +26,9 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 v, i
 // How the waves of a workgroup are laid out: from N and K only, never from M, and the
 // same for every kernel, so that a row of C is computed in the same order whatever else
 // is in the batch and whichever kernel serves it.
-//   wide: 4 waves along N; deep (a long K and too few rows of W to fill the chip with
+//   wide (a short K): 4 waves along N; deep (a long K and too few rows of W to fill the chip with
 //   workgroups of 4): 8 waves split K; otherwise 4 waves split K.
-static inline bool layout_wide(int N, int K) { return N >= 16384 || K < 512; }
+static inline bool layout_wide(int N, int K) { return K < 512; }
 static inline bool layout_deep(int N, int K) { return K >= 2048 && N < 4096; }
 
 // Operands of the product whose workgroups own 16 rows of W and split K among their

@@ -1,7 +1,7 @@
 // C[M,N] = A[M,K] * W[N,K]^T for bfloat16 operands on the matrix cores, float32
 // accumulation, for the shapes where streaming W once is the whole cost: the entry
-// points of the matrix-core products, and the kernels of the wide layout (a very wide N,
-// the output head, or a short K), in which the four waves of a workgroup take different
+// points of the matrix-core products, and the kernels of the wide layout (a short K), in
+// which the four waves of a workgroup take different
 // tiles of 16 rows of W and nobody splits K.  The layouts that split K among a
 // workgroup's waves are gemm_direct.hip's.
 //
@@ -400,12 +400,13 @@ extern "C" int ts_gemm_mfma_bf16(const void* a, const void* w, void* c, int c_ty
 
 // Whether the fused form below takes a product of this shape: at most 16 rows; in the
 // wide layout rows short enough for its staging buffer; in the others at most 16384
-// elements of the residual stream (16 rows of 1024, 4 of 4096), because every workgroup
-// reads them in float32 and with a long K that costs more than the norm kernel saved.
+// elements of the residual stream (16 rows of 1024, 4 of 4096) and a weight of at most
+// 2^24 elements, because every workgroup reads the stream in float32: with a long K or
+// very many workgroups (the output head) that costs more than the norm kernel saved.
 extern "C" int ts_norm_gemm_mfma_fits(int M, int N, int K) {
   if (M < 1 || M > 16 || K <= 0 || K % 8) return 0;
   if (layout_wide(N, K)) return (size_t)M * (K + 8) * 2 <= 140 * 1024;
-  return (int64_t)M * K <= 16384;
+  return (int64_t)M * K <= 16384 && (int64_t)N * K <= (1 << 24);
 }
 
 // 0: 4 waves split K, 1: 8 waves split K, 2: wide (4 waves along N).

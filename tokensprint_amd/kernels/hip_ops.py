@@ -187,22 +187,27 @@ class HipOps:
                        self._stream())
         return out
 
-    # Rows above which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
+    # Rows from which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
     # torch.matmul), as the reference sends every linear layer to its vendor library
-    # (engine/nn/base_layers.py:7-10).  Up to 64 rows the weight-streaming kernels here
-    # are faster, measured inside captured graphs at the Qwen3-0.6B layer shapes, and fuse
-    # the norm before (up to 16 rows) and the SwiGLU after; in the wide layout (the output
-    # head) the library is ahead from 17 rows on.  Its result is bfloat16 (float32
-    # accumulation), as the reference's logits are; float32 results of such a product are
-    # that result widened.
+    # (engine/nn/base_layers.py:7-10).  Measured inside captured graphs at the Qwen3-0.6B
+    # shapes: up to 64 rows the weight-streaming kernels here are faster at the layer
+    # products and fuse the norm before (up to 16 rows) and the SwiGLU after; in the wide
+    # layout (a short K) the library is ahead from 17 rows on, and at the output head (a
+    # very large N, where every one of thousands of workgroups reads all rows of x) from 5.
+    # Its result is bfloat16 (float32 accumulation), as the reference's logits are;
+    # float32 results of such a product are that result widened.
     LIBRARY_ROWS = 65
     LIBRARY_ROWS_WIDE = 17
+    LIBRARY_ROWS_HEAD = 5
+    HEAD_COLUMNS = 16384
 
     def _library_ok(self, x, weight, out_dtype=None):
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             return False
         M = x.shape[0]
         if M >= self.LIBRARY_ROWS:
+            return True
+        if M >= self.LIBRARY_ROWS_HEAD and weight.shape[0] >= self.HEAD_COLUMNS:
             return True
         return (M >= self.LIBRARY_ROWS_WIDE
                 and self.lib.ts_gemm_mfma_layout(weight.shape[0], weight.shape[1]) == 2)
