@@ -70,11 +70,100 @@ __global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
     o[i] = from_f32<TO>(to_f32(xr[i]) * rstd * w[i]);
 }
 
+// The same for a float32 x whose rows are a multiple of 4 wide and fit the registers of a
+// workgroup (the residual stream of every model so far): 16-byte loads, each value read
+// once and kept, and the stores after the loads, which share a counter with them.
+typedef __attribute__((ext_vector_type(4))) float f32x4_rows;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_rows;
+__device__ __forceinline__ f32x4_rows load4(const float* p) { return *(const f32x4_rows*)p; }
+__device__ __forceinline__ f32x4_rows load4(const bf16_t* p) {
+  const bf16x4_rows v = *(const bf16x4_rows*)p;
+  return f32x4_rows{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+__device__ __forceinline__ void store4(float* p, f32x4_rows v) { *(f32x4_rows*)p = v; }
+__device__ __forceinline__ void store4(bf16_t* p, f32x4_rows v) {
+  *(bf16x4_rows*)p = bf16x4_rows{(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+}
+
+template <typename TD, typename TO, bool ADD, int VPT>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(float* __restrict__ x,
+                                                          const TD* __restrict__ delta,
+                                                          const float* __restrict__ w,
+                                                          TO* __restrict__ out, int width,
+                                                          float eps) {
+  __shared__ float scratch[16];
+  const int64_t base = (int64_t)blockIdx.x * width;
+  const int n4 = width / 4;
+  f32x4_rows v[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    v[j] = f32x4_rows{0.f, 0.f, 0.f, 0.f};
+    if (i < n4) {
+      v[j] = load4(x + base + i * 4);
+      if (ADD) {
+        const f32x4_rows d = load4(delta + base + i * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[j][e] += d[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += v[j][e] * v[j][e];
+  }
+  f32x4_rows wv[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    wv[j] = i < n4 ? load4(w + i * 4) : f32x4_rows{0.f, 0.f, 0.f, 0.f};
+  }
+  const float rstd = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i >= n4) continue;
+    if (ADD) store4(x + base + i * 4, v[j]);
+    f32x4_rows o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = v[j][e] * rstd * wv[j][e];
+    store4(out + base + i * 4, o);
+  }
+}
+
+// Launches the vector kernel if the row fits; returns false if it does not.
+template <typename TD, typename TO, bool ADD>
+static bool launch_rmsnorm_vec(float* x, const TD* delta, const float* w, TO* out, int rows,
+                               int width, float eps, hipStream_t stream) {
+  if (width % 4 || width > 256 * 4 * 8) return false;
+  if (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)w | (uintptr_t)out) & 15) return false;
+  const int n4 = width / 4;
+  const int threads = n4 >= 256 ? 256 : (n4 >= 128 ? 128 : 64);
+  const int vpt = (n4 + threads - 1) / threads;
+  if (vpt <= 1)
+    hipLaunchKernelGGL((rmsnorm_vec_kernel<TD, TO, ADD, 1>), dim3(rows), dim3(threads), 0, stream, x, delta, w, out, width, eps);
+  else if (vpt <= 2)
+    hipLaunchKernelGGL((rmsnorm_vec_kernel<TD, TO, ADD, 2>), dim3(rows), dim3(threads), 0, stream, x, delta, w, out, width, eps);
+  else if (vpt <= 4)
+    hipLaunchKernelGGL((rmsnorm_vec_kernel<TD, TO, ADD, 4>), dim3(rows), dim3(threads), 0, stream, x, delta, w, out, width, eps);
+  else
+    hipLaunchKernelGGL((rmsnorm_vec_kernel<TD, TO, ADD, 8>), dim3(rows), dim3(threads), 0, stream, x, delta, w, out, width, eps);
+  return true;
+}
+
 extern "C" int ts_rmsnorm(const void* x, int x_type, const float* w, void* out, int out_type,
                           int rows, int width, float eps, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (width <= 0) TS_FAIL("rmsnorm: width=%d", width);
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  if (x_type == TS_F32) {
+    bool done = false;
+    TS_DISPATCH_TYPE(out_type, TO, done = launch_rmsnorm_vec<float, TO, false>(
+        (float*)x, (const float*)nullptr, w, (TO*)out, rows, width, eps, stream));
+    if (done) {
+      TS_CHECK_LAUNCH("rmsnorm");
+      return 0;
+    }
+  }
   TS_DISPATCH_TYPE(x_type, TX, TS_DISPATCH_TYPE(out_type, TO,
       hipLaunchKernelGGL((rmsnorm_kernel<TX, float, TO, false>), dim3(rows), dim3(threads), 0,
                          stream, (TX*)x, (const float*)nullptr, w, (TO*)out, width, eps)));
@@ -88,6 +177,16 @@ extern "C" int ts_add_rmsnorm(float* resid, const void* delta, int delta_type, c
   if (rows <= 0) return 0;
   if (width <= 0) TS_FAIL("add_rmsnorm: width=%d", width);
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  {
+    bool done = false;
+    TS_DISPATCH_TYPE(delta_type, TD, TS_DISPATCH_TYPE(out_type, TO,
+        done = launch_rmsnorm_vec<TD, TO, true>(resid, (const TD*)delta, w, (TO*)out, rows, width,
+                                                eps, stream)));
+    if (done) {
+      TS_CHECK_LAUNCH("add_rmsnorm");
+      return 0;
+    }
+  }
   TS_DISPATCH_TYPE(delta_type, TD, TS_DISPATCH_TYPE(out_type, TO,
       hipLaunchKernelGGL((rmsnorm_kernel<float, TD, TO, true>), dim3(rows), dim3(threads), 0,
                          stream, resid, (const TD*)delta, w, (TO*)out, width, eps)));
