@@ -38,6 +38,15 @@ TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 8),
         "D": (TINY_D, 3, 32)}   # cfg, seed, page
 
 
+# Two layers of the Qwen3-0.6B shape with a vocabulary wide enough for the output head's
+# own kernels: the widths at which the K-splitting products, their fused norm forms and
+# the fused decode attention serve an engine (the tiny widths above take other kernels).
+# GPU tests only.
+LAYER_E = qwen3_config(hidden=1024, layers=2, heads=16, kv_heads=8, head_dim=128, inter=3072,
+                       vocab=20011, eps=1e-6, theta=1e6, tied=True, max_pos=256)
+GPU_ONLY = {"E": (LAYER_E, 4, 16)}
+
+
 def random_prompt(length, vocab, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (length,), generator=g).tolist()

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import drives
-from helpers import TINY, random_prompt
+from helpers import GPU_ONLY, TINY, random_prompt
 from plain import qwen3_plain as plain
 from tokensprint_amd.engine import ModelRunner
 from tokensprint_amd.engine.assemble import load_model
@@ -19,12 +19,15 @@ pytestmark = pytest.mark.gpu
 TOL = {torch.float32: (1e-4, 2e-5), torch.bfloat16: (3e-2, 3e-2)}
 
 
-@pytest.fixture(scope="module", params=[(n, d) for n in sorted(TINY)
+CONFIGS = {**TINY, **GPU_ONLY}
+
+
+@pytest.fixture(scope="module", params=[(n, d) for n in sorted(CONFIGS)
                                         for d in (torch.float32, torch.bfloat16)],
                 ids=lambda p: f"{p[0]}-{str(p[1]).split('.')[-1]}")
 def setup(request, tmp_path_factory, gpu_device):
     name, dtype = request.param
-    cfg, seed, page = TINY[name]
+    cfg, seed, page = CONFIGS[name]
     d = tmp_path_factory.mktemp(f"tiny{name}")
     write_random_model(d, cfg, seed, dtype)
     pcfg, w = plain.read_model_dir(d)          # the same (rounded) weights, held in float32
