@@ -80,9 +80,10 @@ def test_silu_mul(ops, gpu_device, dtype):
 
 def from_library(M, N, K):
     """Whether a plain bfloat16 product of this shape goes to the vendor library: above 64
-    rows, from 17 rows on where the kernels here lay their waves along N (a short K), and
-    from 5 rows on at a very wide N (the output head)."""
-    return M > 64 or (M > 16 and K < 512) or (M > 4 and N >= 16384)
+    rows, from 17 rows on where the kernels here lay their waves along N (a short K), from
+    5 rows on at a very wide N (the output head), from 9 at weights above 2^23 elements."""
+    return (M > 64 or (M > 16 and K < 512) or (M > 4 and N >= 16384)
+            or (M > 8 and N * K > 2 ** 23))
 
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
@@ -109,6 +110,7 @@ def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
                                    (130, 389, 96), (33, 50, 520), (70, 20000, 64),
                                    (48, 1024, 3072), (64, 1024, 2048), (40, 3000, 1096),
                                    (16, 300, 2056), (23, 520, 640), (4, 20000, 1024),
+                                   (8, 4096, 4096), (12, 4096, 4096),
                                    (6, 20000, 1024)])
 def test_linear_bf16_matrix_core_shapes(ops, gpu_device, out_dtype, M, N, K):
     x = rand((M, K), torch.bfloat16, gpu_device, 17)

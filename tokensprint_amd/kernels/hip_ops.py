@@ -194,12 +194,17 @@ class HipOps:
     # products and fuse the norm before (up to 16 rows) and the SwiGLU after; in the wide
     # layout (a short K) the library is ahead from 17 rows on, and at the output head (a
     # very large N, where every one of thousands of workgroups reads all rows of x) from 5.
+    # At the layer shapes of the 8B and 32B models (weights above 2^23 elements, products
+    # bound by bandwidth, not latency) every workgroup's reading of the rows of x costs
+    # as much as the weights from 16 rows on, and the library is ahead from 9 rows.
     # Its result is bfloat16 (float32 accumulation), as the reference's logits are;
     # float32 results of such a product are that result widened.
     LIBRARY_ROWS = 65
     LIBRARY_ROWS_WIDE = 17
     LIBRARY_ROWS_HEAD = 5
     HEAD_COLUMNS = 16384
+    LIBRARY_ROWS_LARGE = 9
+    LARGE_WEIGHT = 1 << 23
 
     def _library_ok(self, x, weight, out_dtype=None):
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
@@ -208,6 +213,8 @@ class HipOps:
         if M >= self.LIBRARY_ROWS:
             return True
         if M >= self.LIBRARY_ROWS_HEAD and weight.shape[0] >= self.HEAD_COLUMNS:
+            return True
+        if M >= self.LIBRARY_ROWS_LARGE and weight.shape[0] * weight.shape[1] > self.LARGE_WEIGHT:
             return True
         return (M >= self.LIBRARY_ROWS_WIDE
                 and self.lib.ts_gemm_mfma_layout(weight.shape[0], weight.shape[1]) == 2)
