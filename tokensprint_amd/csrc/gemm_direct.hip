@@ -34,7 +34,8 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   __shared__ f32x4 red[(WK - 1) * NW * MT * kWave];
   __shared__ float ss_part[NORM ? WK * 16 : 1];
   const int M = a.M, N = a.N, K = a.K;
-  const int wk = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  // the wave's index as a scalar: the K loop's control is then scalar too
+  const int wk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int r = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
   const int m_base = blockIdx.y * (MT * 16);
@@ -164,14 +165,39 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   constexpr int stride = WK * kStep;
   const int kb0 = wk * kStep;
   Step st[PD];
+  int kb = kb0;
+  // (measured: with one workgroup to a compute unit the waits of the plain loop below,
+  // which let all of a round's loads land before its products, serve better)
+  if (kb0 + (2 * PD - 1) * stride < kfull && gridDim.x * gridDim.y >= 512) {
+    // a long K: rounds in which every buffer is loaded again.  No load in them hangs on a
+    // condition, so the wait before a product is for that product's operands alone (a
+    // load that may or may not have been issued makes the count of those behind it
+    // unknown, and the wait one for nearly all of them).
+    // (the scheduler must not reorder the steps' loads either: they return in the order
+    // issued, and the first step's have to be the oldest)
 #pragma unroll
-  for (int p = 0; p < PD; ++p)
-    if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride);
-  for (int kb = kb0; kb < kfull; kb += PD * stride) {
+    for (int p = 0; p < PD; ++p) {
+      load(st[p], kb0 + p * stride);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    for (; kb + (2 * PD - 1) * stride < kfull; kb += PD * stride) {
+#pragma unroll
+      for (int p = 0; p < PD; ++p) {
+        multiply(st[p]);      // no copy of the step: it would wait for all of it to arrive
+        load(st[p], kb + (p + PD) * stride);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+      if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride);
+  }
+  // the last steps (all of them, for a short K)
+  for (; kb < kfull; kb += PD * stride) {
 #pragma unroll
     for (int p = 0; p < PD; ++p) {
       const int k = kb + p * stride;
-      if (k < kfull) {   // no copy of the step: it would wait for all of it to arrive
+      if (k < kfull) {
         multiply(st[p]);
         if (k + PD * stride < kfull) load(st[p], k + PD * stride);
       }
