@@ -3,14 +3,14 @@
 // short-portion products of up to 64 rows.
 //
 // Nothing is staged: W and A go from global memory straight into the operand layout of
-// v_mfma_f32_16x16x32_bf16, into PD buffers of one step each (a buffer is loaded again
-// as soon as it has been multiplied), so a wave
-// has its whole share of a small product in flight at once and the kernel costs one
-// memory latency, with no barrier before the final sum.  A step is S matrix-core products
-// deep (S * 32 elements of K); S = 4 everywhere except in the fused form with 8 waves,
-// whose float32 operands would not fit the registers twice.  A wave holds up
-// to 4 tiles of 16 rows of A; more rows, or too few workgroups to cover the chip, go to
-// further workgroups along y, which read W again from the second-level cache.
+// v_mfma_f32_16x16x32_bf16, into PD buffers of one step each; a buffer is loaded again as
+// soon as it has been multiplied.  A wave so has its whole share of a small product in
+// flight at once, and the kernel costs one memory latency, with no barrier before the
+// final sum.  A step is S matrix-core products deep (S * 32 elements of K); S = 4
+// everywhere except in the fused form with 8 waves, whose float32 operands would not fit
+// the registers twice.  A wave holds up to 4 tiles of 16 rows of A; more rows, or too few
+// workgroups to cover the chip, go to further workgroups along y, which read W again
+// from the second-level cache.
 //
 // Fused form (at most 16 rows): A is not stored but is the RMSNorm of the residual
 // stream, x = resid_in + delta, A = bf16(x * norm_w) * rsqrt(mean(x^2) + eps).  Every

@@ -54,10 +54,74 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TA* __restrict__ A,
   }
 }
 
+// Up to 16 rows of A (decode steps): a thread per output column and one workgroup of 64
+// threads per 64 columns, so the columns spread over the chip.  A thread walks its row of
+// W in 16-byte pieces (the lines it touches stay in the first-level cache until it has
+// used them up), the rows of A come through scalar loads, the same for every thread.
+// The products of an output element are added in index order, as in the tiled kernel.
+typedef __attribute__((ext_vector_type(4))) float f32x4_fma;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_fma;
+__device__ __forceinline__ f32x4_fma load4_fma(const float* p) { return *(const f32x4_fma*)p; }
+__device__ __forceinline__ f32x4_fma load4_fma(const bf16_t* p) {
+  const bf16x4_fma v = *(const bf16x4_fma*)p;
+  return f32x4_fma{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+template <typename TA, typename TW, typename TC, int MR>
+__global__ __launch_bounds__(64) void gemm_fma_rows_kernel(const TA* __restrict__ A,
+                                                           const TW* __restrict__ W,
+                                                           TC* __restrict__ C, int M, int N, int K) {
+  const int64_t n = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  const TW* wrow = W + min(n, (int64_t)N - 1) * K;
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+  const int k4 = K / 4 * 4;
+  int k = 0;
+  for (; k < k4; k += 4) {
+    const f32x4_fma w = load4_fma(wrow + k);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const f32x4_fma a = load4_fma(A + (int64_t)min(m, M - 1) * K + k);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[m] = fmaf(a[e], w[e], acc[m]);
+    }
+  }
+  for (; k < K; ++k) {
+    const float w = to_f32(wrow[k]);
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+      acc[m] = fmaf(to_f32(A[(int64_t)min(m, M - 1) * K + k]), w, acc[m]);
+  }
+  if (n >= N) return;
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+    if (m < M) C[(int64_t)m * N + n] = from_f32<TC>(acc[m]);
+}
+
+template <typename TA, typename TW, typename TC>
+static void launch_rows(const TA* A, const TW* W, TC* C, int M, int N, int K, hipStream_t stream) {
+  const dim3 grid((N + 63) / 64);
+  if (M == 1)
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 1>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+  else if (M <= 4)
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 4>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 16>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+}
+
 extern "C" int ts_gemm_fma(const void* a, int a_type, const void* w, int w_type, void* c,
                            int c_type, int M, int N, int K, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) TS_FAIL("gemm: K=%d", K);
+  // rows of 4 elements must start on 16 (float32) or 8 (bfloat16) bytes for the row kernel
+  const bool rows_ok = M <= 16 && K % 4 == 0 && (((uintptr_t)a | (uintptr_t)w) & 15) == 0;
+  if (rows_ok) {
+    TS_DISPATCH_TYPE(a_type, TA, TS_DISPATCH_TYPE(w_type, TW, TS_DISPATCH_TYPE(c_type, TC,
+        launch_rows<TA, TW, TC>((const TA*)a, (const TW*)w, (TC*)c, M, N, K, stream))));
+    TS_CHECK_LAUNCH("gemm_fma");
+    return 0;
+  }
   dim3 grid((N + kTile - 1) / kTile, (M + kTile - 1) / kTile);
   if (grid.y > 65535) TS_FAIL("gemm: M=%d too large for one launch", M);
   TS_DISPATCH_TYPE(a_type, TA, TS_DISPATCH_TYPE(w_type, TW, TS_DISPATCH_TYPE(c_type, TC,
