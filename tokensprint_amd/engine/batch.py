@@ -48,6 +48,7 @@ class StepBatch:
     max_q_len: int
     max_ctx_len: int
     plans: dict = field(default_factory=dict)   # kernels cache per-step launch plans here
+    all_rows_wanted: bool = False   # logit_rows is 0..T-1: picking the wanted rows is no work
 
 
 def _align(n: int, a: int = 4) -> int:
@@ -87,7 +88,8 @@ class StaticDecodeBatch:
             entry_of_token=d[o[2]:o[2] + B], q_start=d[o[3]:o[3] + B + 1],
             ctx_len=d[o[4]:o[4] + B], slot_ids=d[o[5]:o[5] + B], logit_rows=d[o[6]:o[6] + B],
             tables=[d[o[7 + g]:o[7 + g] + B * w].view(B, w) for g, w in enumerate(widths)],
-            q_lens=[1] * B, starts=[0] * B, max_q_len=1, max_ctx_len=0)
+            q_lens=[1] * B, starts=[0] * B, max_q_len=1, max_ctx_len=0,
+            all_rows_wanted=True)
         h = self.host.numpy()
         h[:] = 0
         h[o[2]:o[2] + B] = np.arange(B)
@@ -245,4 +247,6 @@ class BatchBuilder:
             tables=[sec(7 + g, B * w).view(B, w) for g, w in enumerate(widths)],
             q_lens=q_lens, starts=starts, max_q_len=max(q_lens),
             max_ctx_len=max(s + n for s, n in zip(starts, q_lens)),
+            all_rows_wanted=R == T and all(e.want == list(range(len(e.tokens)))
+                                           for e in entries),
         )

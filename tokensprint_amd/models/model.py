@@ -86,8 +86,11 @@ class Model:
                 resid, delta, batch, caches[owner], write_cache=run.cache_of is None)
         if batch.num_logit_rows == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=resid.device)
-        resid_rows = ops.gather_rows(resid, batch.logit_rows)
-        delta_rows = None if delta is None else ops.gather_rows(delta, batch.logit_rows)
+        if batch.all_rows_wanted:
+            resid_rows, delta_rows = resid, delta
+        else:
+            resid_rows = ops.gather_rows(resid, batch.logit_rows)
+            delta_rows = None if delta is None else ops.gather_rows(delta, batch.logit_rows)
         fused = self.final_norm.fused_rmsnorm()
         if fused is not None:
             return ops.norm_linear(resid_rows, delta_rows, fused[0], fused[1], self.head.weight,
