@@ -34,11 +34,19 @@ __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirs
 // of 16 lanes of one operand with even rows of the other, v_permlane32_swap the upper 32
 // lanes of one with the lower 32 of the other; fed the same value twice they return the
 // value of each half (pair of rows) in both halves.
+//
+// max2: the larger of two by the NaN-propagating maximum (v_maximum3_f32, which also
+// takes three operands, so two calls in a row are one instruction).  fmaxf would first
+// quiet a signalling NaN in each operand, an instruction per operand and call, which
+// scores (finite products, or -inf from the mask) do not need.
+__device__ __forceinline__ float max2(float a, float b) {
+  return __builtin_elementwise_maximum(a, b);
+}
 __device__ __forceinline__ float col4_max(float v) {
   auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  v = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
   auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float col4_sum(float v) {
   auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -135,9 +143,13 @@ struct TileState {
   static constexpr int DB = HD / 16;
   bf16x8 q[KS];
   f32x4 o[DB];
-  float m, l;
+  float m, l;         // l: this lane's share of the row's sum of weights (row_sum adds the four)
   int pos, lo;        // this lane's row: position and first visible key (pos = -1: no row)
 };
+
+// The sum of weights of a lane's query row: the shares of the four lanes that hold the row.
+template <int HD>
+__device__ __forceinline__ float row_sum(const TileState<HD>& t) { return col4_sum(t.l); }
 
 template <int HD>
 __device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow, bool row_ok,
@@ -183,35 +195,42 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
         st[blk][i] = (key <= t.pos && key >= t.lo) ? st[blk][i] : -INFINITY;
       }
   }
-  float mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
-                   fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+  const float mx = max2(max2(max2(max2(st[0][0], st[0][1]), st[0][2]),
+                             max2(max2(st[0][3], st[1][0]), st[1][1])),
+                        max2(st[1][2], st[1][3]));
   // the scale is positive: the largest score stays the largest
-  const float m_new = fmaxf(t.m, col4_max(mx) * scale_log2);
-  const float m_use = fmaxf(m_new, -1e30f);
+  const float m_new = max2(t.m, col4_max(mx) * scale_log2);
+  const float m_use = max2(m_new, -1e30f);
   const float corr = __builtin_amdgcn_exp2f(t.m - m_use);
-  float ps = 0.f;
+  float ps;
   bf16x8 pv;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i / 4][i % 4], scale_log2, -m_use));
-    ps += p;
+    ps = i ? ps + p : p;
     pv[i] = (bf16_t)p;
   }
-  ps = col4_sum(ps);
+  // the correction is the same in the four lanes of a row, so each lane keeps the sum of
+  // its own keys and the four are added once, at the end
   t.l = t.l * corr + ps;
   t.m = m_new;
+  // far into a long context no row of the tile meets a new largest score in most blocks:
+  // then the sums so far need no rescaling (a wave-uniform test)
+  if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
 #pragma unroll
-  for (int db = 0; db < DB; ++db) {
-    f32x4 acc = t.o[db];
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] *= corr;
-    t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[db], pv, acc, 0, 0, 0);
+      for (int i = 0; i < 4; ++i) t.o[db][i] *= corr;
   }
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+    t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v[db], pv, t.o[db], 0, 0, 0);
 }
 
 template <int HD>
-__device__ __forceinline__ void store_tile(const TileState<HD>& t, bf16_t* out, int g) {
-  const float inv = t.l > 0.f ? 1.f / t.l : 0.f;
+__device__ __forceinline__ void store_tile(const TileState<HD>& t, float sum, bf16_t* out,
+                                           int g) {
+  const float inv = sum > 0.f ? 1.f / sum : 0.f;
 #pragma unroll
   for (int db = 0; db < TileState<HD>::DB; ++db) {
     bf16x4 ov = {(bf16_t)(t.o[db][0] * inv), (bf16_t)(t.o[db][1] * inv),

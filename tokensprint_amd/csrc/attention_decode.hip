@@ -209,7 +209,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
         for (int j = 0; j < 8; ++j) dot += (float)t.q[s][j] * (float)kq[s][j];
       // this wave's partial: one key with weight 1
       t.m = col4_sum(dot) * scale_log2;
-      t.l = 1.f;
+      t.l = g == 0 ? 1.f : 0.f;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const bf16x4 v = *(const bf16x4*)(vrow + db * 16 + g * 4);
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     tile_update<HD>(t, B, kb + stride, scale_log2, kb + stride + 31 <= last && kb + stride >= lo, g);
   }
   f32x4 (&o)[DB] = t.o;
-  float m = t.m, l = t.l;
+  float m = t.m, l = row_sum<HD>(t);
 
   // the waves' partial results (the new key's among them), merged by wave 0 in wave order
   __shared__ float s_ml[NW - 1][kWave][2];
@@ -295,8 +295,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
   if (ma.num_splits == 1) {
     if (!row_ok) return;
-    t.l = l;
-    store_tile<HD>(t, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
+    store_tile<HD>(t, l, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
   } else {
     const int64_t slot = ((int64_t)item * ma.num_splits + split) * 16 + r;
     if (row_ok) {

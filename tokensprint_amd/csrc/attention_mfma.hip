@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
                     kb + kStride + 31 <= pos_first && kb + kStride >= lo_last, g);
   }
   f32x4 (&o)[DB] = t.o;
-  float m = t.m, l = t.l;
+  float m = t.m, l = row_sum<HD>(t);
 
   if (COOP) {   // the four waves' partial results, merged by wave 0 in wave order
     __shared__ float s_ml[3][kWave][2];
@@ -131,8 +131,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
   if (args.num_splits == 1) {
     if (!row_ok) return;
-    t.l = l;
-    store_tile<HD>(t, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
+    store_tile<HD>(t, l, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
   } else {
     const int64_t slot = ((int64_t)item * args.num_splits + split) * 16 + r;
     if (row_ok) {

@@ -80,8 +80,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
 
 #pragma unroll
   for (int j = 0; j < TPW; ++j) {
+    const float sum = row_sum<HD>(ts[j]);        // by all lanes: it crosses lanes
     if (ts[j].pos < 0) continue;
-    store_tile<HD>(ts[j], (bf16_t*)a.out + ((int64_t)(tok0 + j * tq + ti) * a.nq + head) * HD, g);
+    store_tile<HD>(ts[j], sum,
+                   (bf16_t*)a.out + ((int64_t)(tok0 + j * tq + ti) * a.nq + head) * HD, g);
   }
 }
 
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   struct Fetched {
     bf16x8 k[KQ];
     bf16x4 v[VQ];
-    bool kvalid[KQ], vvalid[VQ];                // wave-uniform
+    bool kvalid[KQ], vvalid[VQ];                // wave-uniform but for the head size's tail
   };
   Fetched ring[kAhead];
   // address = head base + page * page stride (scalar) + position in page (scalar)
@@ -169,7 +171,10 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   const int64_t k_page_stride = (int64_t)a.nkv * P * HD, v_page_stride = k_page_stride;
   const bf16_t* k_head = kp + (int64_t)kvh * P * HD;
   const bf16_t* v_head = vp + (int64_t)kvh * HD * P;
-  int k_lane[KQ], v_lane[VQ], k_blk[KQ], v_blk[VQ];
+  // in bytes and unsigned: added to a scalar base as a 32-bit offset, without 64-bit
+  // lane arithmetic (a page of one head is far below 4 GiB)
+  unsigned k_lane[KQ], v_lane[VQ];
+  int k_blk[KQ], v_blk[VQ];
   bool k_dim_ok[KQ];
 #pragma unroll
   for (int i = 0; i < KQ; ++i) {
@@ -177,14 +182,20 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
     const int s0 = q % KS;
     k_blk[i] = q / KS;
     k_dim_ok[i] = KS * 32 == HD || g * 8 * KS + s0 * 8 < HD;
-    k_lane[i] = r * HD + min(g * 8 * KS + s0 * 8, HD - 8);
+    k_lane[i] = 2u * (r * HD + min(g * 8 * KS + s0 * 8, HD - 8));
   }
 #pragma unroll
   for (int i = 0; i < VQ; ++i) {
     const int q = vEven ? wave + 4 * i : min(wave + 4 * i, 2 * DB - 1);
     v_blk[i] = q / DB;
-    v_lane[i] = ((q % DB) * 16 + r) * P + g * 4;
+    v_lane[i] = 2u * (((q % DB) * 16 + r) * P + g * 4);
   }
+  // the offset as the load sees it: opaque, so that it stays a 32-bit register beside the
+  // scalar base instead of being widened once, outside the loop, into a register pair
+  auto lane_offset = [](unsigned off) {
+    asm volatile("" : "+v"(off));
+    return off;
+  };
   auto fetch = [&](Fetched& f, int kb) {
     const int in_page = kb & (P - 1);             // a block of 16 keys never straddles a page
     const int page0 = cur.next0, page1 = cur.next1;
@@ -196,16 +207,18 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
 #pragma unroll
     for (int i = 0; i < KQ; ++i) {
       f.kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
-      f.k[i] = *(const bf16x8*)((k_blk[i] ? kb1 : kb0) + k_lane[i]);
+      f.k[i] = *(const bf16x8*)((const char*)(k_blk[i] ? kb1 : kb0) + lane_offset(k_lane[i]));
     }
 #pragma unroll
     for (int i = 0; i < VQ; ++i) {
       f.vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
-      f.v[i] = *(const bf16x4*)((v_blk[i] ? vb1 : vb0) + v_lane[i]);
+      f.v[i] = *(const bf16x4*)((const char*)(v_blk[i] ? vb1 : vb0) + lane_offset(v_lane[i]));
     }
     cur.start(kb + 32);
   };
-  auto stash = [&](const Fetched& f, int buf) {    // registers -> LDS, operand layout
+  // registers -> LDS, operand layout.  (Blanking under a branch, taken only by the last
+  // block of a context, was measured: slower than the selects it saves.)
+  auto stash = [&](const Fetched& f, int buf) {
 #pragma unroll
     for (int i = 0; i < KQ; ++i)
       if (kEven || wave + 4 * i < 2 * KS)
@@ -246,8 +259,9 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
       buf ^= 1;
     }
   }
+  const float sum = row_sum<HD>(t);                // by all lanes: it crosses lanes
   if (row_ok)
-    store_tile<HD>(t, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+    store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
 }
 
 // Query tiles per wavefront: as many as the register file holds accumulators for.
