@@ -173,7 +173,12 @@ __device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow,
 // way.  scale_log2 = softmax scale * log2(e); m is kept in that unit.  A row that has
 // seen no key yet has m = -inf; the exponentials take a finite stand-in for it, which
 // makes all of them 0 without a special case.
-template <int HD>
+//
+// LAZY: the sums so far are rescaled only if some row of the tile met a new largest score
+// (a wave-uniform branch).  Far into a long context most blocks bring none.  For kernels
+// whose loads of the next block are in flight across this call the branch costs more
+// than it saves (the waits at its join are for all of them).
+template <int HD, bool LAZY = false>
 __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>& b, int kb,
                                             float scale_log2, bool interior, int g) {
   constexpr int KS = TileState<HD>::KS, DB = TileState<HD>::DB;
@@ -214,9 +219,7 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
   // its own keys and the four are added once, at the end
   t.l = t.l * corr + ps;
   t.m = m_new;
-  // far into a long context no row of the tile meets a new largest score in most blocks:
-  // then the sums so far need no rescaling (a wave-uniform test)
-  if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+  if (!LAZY || __builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll

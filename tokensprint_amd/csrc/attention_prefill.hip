@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
           for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = k_lds[buf][blk * KS + s0][lane];
 #pragma unroll
         for (int db = 0; db < DB; ++db) b.v[db] = v_lds[buf][db][lane];
-        tile_update<HD>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
+        tile_update<HD, true>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
       }
       if (kb + 32 <= pos_last) stash(ring[(p + 1) % kAhead], buf ^ 1);
       __syncthreads();
