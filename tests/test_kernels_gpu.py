@@ -192,6 +192,82 @@ def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
         assert excess <= 0, f"error exceeds the rounding bound by {float(excess):.3e}"
 
 
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("M,W,K,N", [(8, 1024, 2048, 4096), (1, 1024, 3072, 6144), (64, 1024, 2048, 4096),
+                                     (33, 520, 1096, 1392), (16, 1000, 2056, 112), (17, 4096, 512, 160),
+                                     (7, 2048, 4096, 528), (40, 1000, 520, 2000)])
+def test_linear_into_stream_then_norm_linear(ops, gpu_device, silu, M, W, K, N):
+    """The norm split over two products (bfloat16 only): the first adds bf16(x Wo^T) into
+    the stream [M, W] in place and prepares the rows, the second is norm_linear over them.
+    Against float64 from the stream the first one must leave, with norm_linear's bound."""
+    from tokensprint_amd.kernels.stream import NormHint, PreparedRows
+    bf = torch.bfloat16
+    resid = rand((M, W), torch.float32, gpu_device, 50)
+    x = rand((M, K), bf, gpu_device, 51)
+    wo = rand((W, K), bf, gpu_device, 52, scale=0.05)
+    nw = 1 + 0.1 * rand((W,), torch.float32, gpu_device, 53)
+    w = rand((N, W), bf, gpu_device, 54, scale=0.05)
+    hint = NormHint(nw, 1e-5, w, silu)
+    r = resid.clone()
+    prepared = ops.linear_into_stream(x, wo, r, hint)
+    assert isinstance(prepared, PreparedRows), "these shapes are ones the fused kernels take"
+    delta = (x.double() @ wo.double().T)
+    # the product is rounded to bfloat16 (unit roundoff 2^-8) before the add, as the
+    # separate kernels do
+    eps = 2.0 ** -9
+    dnoise = 2 * eps * delta.abs() + 4 * 2.0 ** -24 * (K ** 0.5) * float(
+        x.double().pow(2).mean().sqrt() * wo.double().pow(2).mean().sqrt())
+    assert ((r.double() - (resid.double() + delta)).abs() <= 1.01 * dnoise + 1e-6).all()
+    xs = r.double()
+    assert torch.allclose(prepared.sumsq.double().sum(0), xs.pow(2).sum(-1), rtol=1e-5)
+    torch.testing.assert_close(prepared.rows.float(), (r * nw).to(bf).float(), rtol=2 ** -7, atol=1e-30)
+    h = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
+    y = h @ w.double().T
+    dot_noise = eps * (W ** 0.5) * float(h.pow(2).mean().sqrt() * w.double().pow(2).mean().sqrt())
+    noise = 4 * (dot_noise + eps * y.abs())
+    if silu:
+        g, u = y[:, :N // 2], y[:, N // 2:]
+        ref = torch.nn.functional.silu(g) * u
+        sg = torch.nn.functional.silu(g).abs()
+        bound = 1.2 * (u.abs() + noise[:, N // 2:]) * noise[:, :N // 2] + sg * noise[:, N // 2:] \
+            + 4 * eps * ref.abs()
+    else:
+        ref, bound = y, noise
+    out, r_out = ops.norm_linear(r, prepared, nw, 1e-5, w, bf, silu_mul=silu)
+    assert r_out is r
+    # The bound is four standard deviations of the rounding noise: it is for the number of
+    # results that the other product tests hold, so it is applied to the first 16 rows;
+    # the rest is covered by the next check, bit for bit.
+    excess = ((out.double() - ref).abs() - bound)[:16].max()
+    assert excess <= 0, f"error exceeds the rounding bound by {float(excess):.3e}"
+    # a row's result does not depend on the other rows of the step, nor on the tile of
+    # rows it lands in: eight rows at a time give the same bits
+    for m0 in range(0, M, 8):
+        r8 = resid[m0:m0 + 8].clone()
+        p8 = ops.linear_into_stream(x[m0:m0 + 8].contiguous(), wo, r8, hint)
+        out8, _ = ops.norm_linear(r8, p8, nw, 1e-5, w, bf, silu_mul=silu)
+        assert torch.equal(r8, r[m0:m0 + 8]) and torch.equal(out8, out[m0:m0 + 8]), m0
+    # rows prepared for one norm are refused by another
+    with pytest.raises(ValueError):
+        ops.norm_linear(r, prepared, nw.clone(), 1e-5, w, bf, silu_mul=silu)
+
+
+def test_linear_into_stream_declines_what_it_cannot_fuse(ops, gpu_device):
+    from tokensprint_amd.kernels.stream import NormHint
+    bf = torch.bfloat16
+    nw = torch.ones(1024, device=gpu_device)
+    w = rand((4096, 1024), bf, gpu_device, 1)
+    wo = rand((1024, 2048), bf, gpu_device, 2)
+    for M, dt in ((65, bf), (8, torch.float32)):
+        x = rand((M, 2048), dt, gpu_device, 3)
+        r = rand((M, 1024), torch.float32, gpu_device, 4)
+        before = r.clone()
+        assert ops.linear_into_stream(x, wo if dt == bf else wo.float(), r, NormHint(nw, 1e-6, w)) is None
+        assert torch.equal(r, before)
+    assert ops.linear_into_stream(rand((8, 2048), bf, gpu_device, 3), wo,
+                                  rand((8, 1024), torch.float32, gpu_device, 4), None) is None
+
+
 def test_linear_rows_do_not_depend_on_the_batch(ops, gpu_device):
     x = rand((70, 200), torch.float32, gpu_device, 9)
     w = rand((150, 200), torch.float32, gpu_device, 10)

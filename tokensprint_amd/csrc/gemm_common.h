@@ -43,8 +43,23 @@ struct DirectArgs {
   float* resid_out;         // fused form: [M, K], written by workgroup column 0
   int M, N, K;
   float eps;
+  // tail form (resid set): nothing goes to C; the product, rounded to bfloat16, is added
+  // to the residual stream in place, and the new stream is handed on prepared for the
+  // RMSNorm that follows: rows x * tail_w, and per row the sum of x^2 over this
+  // workgroup's 16 columns
+  float* resid;             // [M, N]
+  const float* tail_w;      // [N]
+  bf16_t* prepared;         // [M, N] out
+  float* sumsq_out;         // [ceil(N / 16)][M] out
+  // scaled form (sumsq set): A holds such prepared rows; C's rows are divided by the
+  // root mean square that the slices of sums of squares give
+  const float* sumsq;       // [parts][M]
+  int parts;
 };
 
 // Launches it; `norm` (the fused form) takes at most 16 rows.  Returns 0 or -1 with the
 // error text set.
 int gemm_direct_launch(const DirectArgs& a, int c_type, bool pair, bool norm, hipStream_t stream);
+// Whether the tail and the scaled form take a product of this shape (up to 64 rows).
+bool gemm_direct_tail_fits(int M, int N, int K);
+bool gemm_direct_scaled_fits(int M, int N, int K, bool pair);

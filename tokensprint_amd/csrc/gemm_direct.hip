@@ -21,18 +21,34 @@
 // a store inside the loop would share the loads' counter and make every wait for an
 // operand a wait for everything in flight.
 //
+// Tail and scaled form (up to 64 rows): the same norm split over two products.  The
+// product that ends a sub-layer (TAIL) adds its result to the residual stream in place,
+// x = resid + bf16(A W^T), and leaves for the product that follows the rows x * norm_w in
+// bfloat16 and, per workgroup column, each row's sum of x^2 over its 16 columns.  That
+// product (SCALED) is a plain one over the prepared rows; its waves add the slices of a
+// row's sum of squares, in a fixed order, while their operands are on the way, and the
+// row factor is applied to the sums at the end.  No workgroup reads the float32 stream
+// but the one that updates its own 16 columns of it.
+//
 // The K split and the order of the final sum are those of the layout rule, so a row's
 // result is bit for bit the same for any number of rows and any tile it lands in.
+#include <type_traits>
 #include "gemm_common.h"
 
-template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD>
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD, bool SCALED = false,
+          bool TAIL = false>
 __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   static_assert(!NORM || MT == 1, "the fused form holds one tile of rows");
+  static_assert(!(NORM && SCALED) && !(TAIL && (NORM || SCALED || PAIR)), "one form at a time");
+  // slices of the sums of squares a lane adds per tile (16 registers in all)
+  constexpr int kPartLoads = SCALED ? 16 / MT : 1;
   constexpr int kStep = S * 32;          // K elements of one step
   constexpr int kLane = S * 8;           // of which a lane holds this many, contiguous
   constexpr int NW = PAIR ? 2 : 1;
   __shared__ f32x4 red[(WK - 1) * NW * MT * kWave];
-  __shared__ float ss_part[NORM ? WK * 16 : 1];
+  __shared__ float ss_part[(NORM || SCALED) ? WK * MT * 16 : 1];
   const int M = a.M, N = a.N, K = a.K;
   // the wave's index as a scalar: the K loop's control is then scalar too
   const int wk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -71,6 +87,31 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
       cd = *(const bf16x8*)(dbase + c_off);
     }
   }
+
+  // tail form: this lane's four columns of the stream and of the next norm's weight,
+  // asked for first by every wave (no load hangs on a condition), used by wave 0 last
+  const int tail_n = min(n0 + g * 4, max(N - 4, 0));
+  f32x4 tail_x[TAIL ? MT : 1], tail_w4 = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (TAIL) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      tail_x[mt] = *(const f32x4*)(a.resid + (int64_t)min(m_base + mt * 16 + r, M - 1) * N + tail_n);
+    tail_w4 = *(const f32x4*)(a.tail_w + tail_n);
+  }
+  // scaled form: slice j of a row's sum of squares goes to wave (j / 4) % WK, lane group
+  // j % 4; a slice past the last reads the last again and is dropped
+  float part[MT][kPartLoads];
+  auto load_parts = [&]() {
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < kPartLoads; ++i) {
+          const int j = (i * WK + wk) * 4 + g;
+          part[mt][i] = a.sumsq[(int64_t)min(j, a.parts - 1) * M + min(m_base + mt * 16 + r, M - 1)];
+        }
+    }
+  };
 
   f32x4 acc[NW][MT];
 #pragma unroll
@@ -180,6 +221,8 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
       load(st[p], kb0 + p * stride);
       __builtin_amdgcn_sched_barrier(0);
     }
+    load_parts();
+    __builtin_amdgcn_sched_barrier(0);
     for (; kb + (2 * PD - 1) * stride < kfull; kb += PD * stride) {
 #pragma unroll
       for (int p = 0; p < PD; ++p) {
@@ -191,6 +234,7 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
 #pragma unroll
     for (int p = 0; p < PD; ++p)
       if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride);
+    load_parts();
   }
   // the last steps (all of them, for a short K)
   for (; kb < kfull; kb += PD * stride) {
@@ -232,6 +276,19 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
     ss += __shfl_xor(ss, 32, kWave);
     if (g == 0) ss_part[wk * 16 + r] = ss;
   }
+  if constexpr (SCALED) {
+    // the row's squares: this lane's slices in order, the four lane groups, then (below)
+    // the waves in order
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < kPartLoads; ++i) sq += ((i * WK + wk) * 4 + g < a.parts) ? part[mt][i] : 0.f;
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0) ss_part[(wk * MT + mt) * 16 + r] = sq;
+    }
+  }
   if (WK > 1) {   // partial sums of the K splits, added in split order
     if (wk > 0) {
 #pragma unroll
@@ -250,16 +307,47 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
         for (int mt = 0; mt < MT; ++mt)
           acc[w][mt] += red[(((k2 - 1) * NW + w) * MT + mt) * kWave + lane];
   }
-  float rstd = 1.f;
-  if constexpr (NORM) {
-    float total = 0.f;
+  float rstd[MT];
 #pragma unroll
-    for (int k2 = 0; k2 < WK; ++k2) total += ss_part[k2 * 16 + r];
-    rstd = rsqrtf(total / (float)K + a.eps);
+  for (int mt = 0; mt < MT; ++mt) {
+    rstd[mt] = 1.f;
+    if constexpr (NORM || SCALED) {
+      float total = 0.f;
+#pragma unroll
+      for (int k2 = 0; k2 < WK; ++k2) total += ss_part[(k2 * MT + mt) * 16 + r];
+      rstd[mt] = rsqrtf(total / (float)K + a.eps);
+    }
   }
 
   // lane holds D[n = n0 + g*4 + t][m = tile*16 + r], t = 0..3
   const int n = n0 + g * 4;
+  if constexpr (TAIL) {
+    const bool n_ok = n < N;                 // N is a multiple of 4 here
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = m_base + mt * 16 + r;
+      f32x4 x = tail_x[mt];
+      float sq = 0.f;
+      bf16x4_t h;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        // the product rounded to the activation type first, as the unfused path stores it
+        x[t] += (float)(bf16_t)acc[0][mt][t];
+        sq += x[t] * x[t];
+        h[t] = (bf16_t)(x[t] * tail_w4[t]);
+      }
+      const bool ok = n_ok && m < M;
+      if (ok) {
+        *(f32x4*)(a.resid + (int64_t)m * N + n) = x;
+        *(bf16x4_t*)(a.prepared + (int64_t)m * N + n) = h;
+      }
+      sq = ok ? sq : 0.f;
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0 && m < M) a.sumsq_out[(int64_t)blockIdx.x * M + m] = sq;
+    }
+    return;
+  }
   if (n >= N) return;
   TC* C = (TC*)a.C;
 #pragma unroll
@@ -267,16 +355,16 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
     const int m = m_base + mt * 16 + r;
     if (m >= M) continue;
     f32x4 v = acc[0][mt];
-    if (NORM) {
+    if (NORM || SCALED) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) v[t] *= rstd;
+      for (int t = 0; t < 4; ++t) v[t] *= rstd[mt];
     }
     if (PAIR) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         // the two products are rounded to the activation type first, as the unfused
         // path stores them, then silu(gate) * up in float32
-        const float gt = (float)(bf16_t)v[t], up = (float)(bf16_t)(acc[1][mt][t] * rstd);
+        const float gt = (float)(bf16_t)v[t], up = (float)(bf16_t)(acc[1][mt][t] * rstd[mt]);
         v[t] = gt / (1.f + expf(-gt)) * up;
       }
     }
@@ -284,10 +372,11 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   }
 }
 
-template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD>
+template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD, bool SCALED = false,
+          bool TAIL = false>
 static void launch(const DirectArgs& a, hipStream_t stream) {
   dim3 grid((a.N + 15) / 16, (a.M + MT * 16 - 1) / (MT * 16));
-  hipLaunchKernelGGL((gemm_direct_kernel<MT, WK, TC, PAIR, NORM, S, PD>), grid,
+  hipLaunchKernelGGL((gemm_direct_kernel<MT, WK, TC, PAIR, NORM, S, PD, SCALED, TAIL>), grid,
                      dim3(WK * kWave), 0, stream, a);
 }
 
@@ -314,6 +403,32 @@ static int dispatch(const DirectArgs& a, bool norm, hipStream_t stream) {
     return 0;
   }
   const int mt = tiles_per_workgroup(a.M, a.N, PAIR ? 2 : 4);
+  if (a.sumsq) {
+    if (deep) {
+      if (mt == 1) launch<1, 8, TC, PAIR, false, 4, 4, true>(a, stream);
+      else if (mt == 2) launch<2, 8, TC, PAIR, false, 4, 3, true>(a, stream);
+      else if constexpr (!PAIR) launch<4, 8, TC, PAIR, false, 4, 2, true>(a, stream);
+    } else {
+      if (mt == 1) launch<1, 4, TC, PAIR, false, 4, 4, true>(a, stream);
+      else if (mt == 2) launch<2, 4, TC, PAIR, false, 4, 3, true>(a, stream);
+      else if constexpr (!PAIR) launch<4, 4, TC, PAIR, false, 4, 2, true>(a, stream);
+    }
+    return 0;
+  }
+  if constexpr (!PAIR && std::is_same<TC, bf16_t>::value) {
+    if (a.resid) {
+      if (deep) {
+        if (mt == 1) launch<1, 8, TC, false, false, 4, 4, false, true>(a, stream);
+        else if (mt == 2) launch<2, 8, TC, false, false, 4, 3, false, true>(a, stream);
+        else launch<4, 8, TC, false, false, 4, 2, false, true>(a, stream);
+      } else {
+        if (mt == 1) launch<1, 4, TC, false, false, 4, 4, false, true>(a, stream);
+        else if (mt == 2) launch<2, 4, TC, false, false, 4, 3, false, true>(a, stream);
+        else launch<4, 4, TC, false, false, 4, 2, false, true>(a, stream);
+      }
+      return 0;
+    }
+  }
   if (deep) {
     if (mt == 1) launch<1, 8, TC, PAIR, false, 4, 4>(a, stream);
     else if (mt == 2) launch<2, 8, TC, PAIR, false, 4, 3>(a, stream);
@@ -326,9 +441,25 @@ static int dispatch(const DirectArgs& a, bool norm, hipStream_t stream) {
   return 0;
 }
 
+bool gemm_direct_tail_fits(int M, int N, int K) {
+  return M >= 1 && M <= 64 && !layout_wide(N, K) && K > 0 && K % 8 == 0 && N % 4 == 0;
+}
+
+bool gemm_direct_scaled_fits(int M, int N, int K, bool pair) {
+  if (M < 1 || M > 64 || layout_wide(N, K) || K <= 0 || K % 8) return false;
+  const int mt = tiles_per_workgroup(M, N, pair ? 2 : 4);
+  const int waves = layout_deep(N, K) ? 8 : 4;
+  return (K + 15) / 16 <= (16 / mt) * 4 * waves;     // the slices its lanes hold
+}
+
 int gemm_direct_launch(const DirectArgs& a, int c_type, bool pair, bool norm,
                        hipStream_t stream) {
   if (layout_wide(a.N, a.K)) TS_FAIL("gemm_direct: not for the wide layout (N=%d, K=%d)", a.N, a.K);
+  if (a.resid && (norm || pair || a.sumsq || c_type != TS_BF16 || !gemm_direct_tail_fits(a.M, a.N, a.K)))
+    TS_FAIL("gemm_direct: the tail form does not take this product (M=%d, N=%d, K=%d)", a.M, a.N, a.K);
+  if (a.sumsq && (norm || a.parts != (a.K + 15) / 16 || !gemm_direct_scaled_fits(a.M, a.N, a.K, pair)))
+    TS_FAIL("gemm_direct: the scaled form does not take this product (M=%d, N=%d, K=%d, %d slices)",
+            a.M, a.N, a.K, a.parts);
   if (a.K <= 0 || a.K % 8) TS_FAIL("gemm_direct: K=%d must be a positive multiple of 8", a.K);
   if (norm && a.M > 16) TS_FAIL("gemm_direct: the fused form takes at most 16 rows, got %d", a.M);
   if ((a.M + 15) / 16 > 65535) TS_FAIL("gemm_direct: M=%d too large", a.M);

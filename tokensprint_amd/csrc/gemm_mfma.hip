@@ -459,3 +459,50 @@ extern "C" int ts_norm_gemm_mfma_bf16(const float* resid_in, const void* delta, 
   TS_CHECK_LAUNCH("norm_gemm_mfma");
   return 0;
 }
+
+// The norm split over two products, for up to 64 rows (see gemm_direct.hip).
+//
+// ts_gemm_tail_bf16: resid[M, N] += bf16(A[M, K] W[N, K]^T) in place (float32), and for
+// the RMSNorm with weight norm_w that follows: prepared[M, N] = bf16(resid * norm_w) and
+// sumsq[ceil(N / 16)][M], each row's sum of squares of resid over 16 columns.
+extern "C" int ts_gemm_tail_fits(int M, int N, int K) { return gemm_direct_tail_fits(M, N, K); }
+
+extern "C" int ts_gemm_tail_bf16(const void* a, const void* w, float* resid, const float* norm_w,
+                                 void* prepared, float* sumsq, int M, int N, int K,
+                                 hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!gemm_direct_tail_fits(M, N, K))
+    TS_FAIL("gemm_tail: M=%d, N=%d, K=%d is not a product the tail form takes", M, N, K);
+  if (((uintptr_t)a | (uintptr_t)w | (uintptr_t)resid | (uintptr_t)norm_w) & 15)
+    TS_FAIL("gemm_tail: operands must be 16-byte aligned");
+  if (((uintptr_t)prepared) & 7) TS_FAIL("gemm_tail: the prepared rows must be 8-byte aligned");
+  if (!a || !w || !resid || !norm_w || !prepared || !sumsq) TS_FAIL("gemm_tail: null operand");
+  DirectArgs da = {};
+  da.A = (const bf16_t*)a; da.W = (const bf16_t*)w; da.M = M; da.N = N; da.K = K;
+  da.resid = resid; da.tail_w = norm_w; da.prepared = (bf16_t*)prepared; da.sumsq_out = sumsq;
+  if (gemm_direct_launch(da, TS_BF16, false, false, stream)) return -1;
+  TS_CHECK_LAUNCH("gemm_tail");
+  return 0;
+}
+
+// ts_gemm_scaled_bf16: C[M, N] = (prepared[M, K] W[N, K]^T) * rsqrt(sum_j sumsq[j][m] / K + eps)
+// for sumsq[ceil(K / 16)][M]; pair as in ts_gemm_mfma_bf16.
+extern "C" int ts_gemm_scaled_fits(int M, int N, int K, int pair) {
+  return gemm_direct_scaled_fits(M, N, K, pair != 0);
+}
+
+extern "C" int ts_gemm_scaled_bf16(const void* prepared, const float* sumsq, float eps,
+                                   const void* w, void* c, int c_type, int M, int N, int K,
+                                   int pair, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!gemm_direct_scaled_fits(M, N, K, pair != 0))
+    TS_FAIL("gemm_scaled: M=%d, N=%d, K=%d is not a product the scaled form takes", M, N, K);
+  if (((uintptr_t)prepared | (uintptr_t)w) & 15) TS_FAIL("gemm_scaled: operands must be 16-byte aligned");
+  if (!prepared || !sumsq || !w || !c) TS_FAIL("gemm_scaled: null operand");
+  DirectArgs da = {};
+  da.A = (const bf16_t*)prepared; da.W = (const bf16_t*)w; da.C = c; da.M = M; da.N = N; da.K = K;
+  da.sumsq = sumsq; da.parts = (K + 15) / 16; da.eps = eps;
+  if (gemm_direct_launch(da, c_type, pair != 0, false, stream)) return -1;
+  TS_CHECK_LAUNCH("gemm_scaled");
+  return 0;
+}

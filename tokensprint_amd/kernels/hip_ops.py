@@ -14,6 +14,7 @@ from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
 import torch
 
 from tokensprint_amd.kernels.build import build, find_library
+from tokensprint_amd.kernels.stream import NormHint, PreparedRows
 
 ABI_VERSION = 1
 _TYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -209,15 +210,17 @@ class HipOps:
     def _library_ok(self, x, weight, out_dtype=None):
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
             return False
-        M = x.shape[0]
+        return self._library_rows(x.shape[0], weight.shape[0], weight.shape[1])
+
+    def _library_rows(self, M, N, K):
+        """Whether a bfloat16 product of M rows with a weight [N, K] is the library's."""
         if M >= self.LIBRARY_ROWS:
             return True
-        if M >= self.LIBRARY_ROWS_HEAD and weight.shape[0] >= self.HEAD_COLUMNS:
+        if M >= self.LIBRARY_ROWS_HEAD and N >= self.HEAD_COLUMNS:
             return True
-        if M >= self.LIBRARY_ROWS_LARGE and weight.shape[0] * weight.shape[1] > self.LARGE_WEIGHT:
+        if M >= self.LIBRARY_ROWS_LARGE and N * K > self.LARGE_WEIGHT:
             return True
-        return (M >= self.LIBRARY_ROWS_WIDE
-                and self.lib.ts_gemm_mfma_layout(weight.shape[0], weight.shape[1]) == 2)
+        return M >= self.LIBRARY_ROWS_WIDE and self.lib.ts_gemm_mfma_layout(N, K) == 2
 
     @staticmethod
     def _mfma_ok(x, weight):
@@ -226,6 +229,53 @@ class HipOps:
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and x.shape[1] % 8 == 0)
 
+    def linear_into_stream(self, x, weight, resid, hint):
+        """The product that ends a sub-layer, told what follows (`hint`, a NormHint).
+        Where one kernel can do it (bfloat16, up to 64 rows, both products among those
+        this provider keeps from the library): resid += bf16(x W^T) in place, and the
+        PreparedRows for the hinted norm and product are returned, to be passed on as
+        the stream's delta.  Otherwise None, and nothing has been done: the caller runs
+        `linear` and passes its result on."""
+        if hint is None or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
+                or hint.weight.dtype != torch.bfloat16:
+            return None
+        self._check("x", x, torch.bfloat16, ndim=2)
+        self._check("weight", weight, torch.bfloat16, ndim=2)
+        M, K = x.shape
+        N = weight.shape[0]
+        if weight.shape[1] != K:
+            raise ValueError(f"linear_into_stream: x has {K} columns, weight has {weight.shape[1]}")
+        next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
+        if hint.weight.shape[1] != N or self._library_rows(M, N, K) \
+                or self._library_rows(M, next_n, N) \
+                or self.lib.ts_gemm_tail_fits(M, N, K) != 1 \
+                or self.lib.ts_gemm_scaled_fits(M, next_n, N, int(hint.silu_mul)) != 1:
+            return None
+        self._check("resid", resid, torch.float32, shape=(M, N))
+        self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
+        rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
+        sumsq = torch.empty((N + 15) // 16, M, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_gemm_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
+                   _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, self._stream())
+        return PreparedRows(rows, sumsq, hint)
+
+    def _prepared_linear(self, resid, prepared, norm_weight, eps, weight, out_dtype, silu_mul):
+        hint = prepared.hint
+        if hint.norm_weight is not norm_weight or hint.eps != eps or hint.weight is not weight \
+                or hint.silu_mul != silu_mul:
+            raise ValueError("norm_linear: the rows were prepared for another norm or product")
+        M, K = prepared.rows.shape
+        if resid.shape != (M, K):
+            raise ValueError("norm_linear: prepared rows and stream differ in shape")
+        N = weight.shape[0] // 2 if silu_mul else weight.shape[0]
+        if out_dtype not in (torch.bfloat16, torch.float32) or (silu_mul and out_dtype != torch.bfloat16):
+            raise ValueError(f"norm_linear: prepared rows cannot give {out_dtype}")
+        out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        self._call(self.lib.ts_gemm_scaled_bf16, _ptr(prepared.rows), _ptr(prepared.sumsq),
+                   c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                   int(silu_mul), self._stream())
+        return out, resid
+
     def norm_linear(self, resid, delta, norm_weight, eps, weight, out_dtype, silu_mul=False):
         """(RMSNorm(resid + delta) W^T, resid + delta): the residual add, the norm and
         the product in one kernel where it can be (bfloat16 weights, at most 16 rows);
@@ -233,6 +283,9 @@ class HipOps:
         the weight is [Wg; Wu] and the result silu(h Wg^T) * (h Wu^T).  The returned
         residual stream may or may not be the tensor passed in."""
         self._check("resid", resid, torch.float32, ndim=2)
+        if isinstance(delta, PreparedRows):     # already added in, by linear_into_stream
+            return self._prepared_linear(resid, delta, norm_weight, eps, weight, out_dtype,
+                                         silu_mul)
         M, K = resid.shape
         self._check("weight", weight, self._FLOATS, ndim=2)
         if weight.shape[1] != K:

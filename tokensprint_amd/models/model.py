@@ -82,8 +82,13 @@ class Model:
         delta = None
         for r, run in enumerate(self.order):
             owner = r if run.cache_of is None else run.cache_of
+            # what reads the stream after this run: the next run's block (the final norm
+            # and the head take a plain delta)
+            next_hint = self.blocks[self.order[r + 1].layer].entry_hint() \
+                if r + 1 < len(self.order) else None
             resid, delta = self.blocks[run.layer].forward(
-                resid, delta, batch, caches[owner], write_cache=run.cache_of is None)
+                resid, delta, batch, caches[owner], write_cache=run.cache_of is None,
+                next_hint=next_hint)
         if batch.num_logit_rows == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=resid.device)
         if batch.all_rows_wanted:

@@ -68,17 +68,21 @@ class GroupedQueryAttention(Mixer):
         return PagedKVNeed(self.nkv, self.hd, self.window)
 
     # -- step
-    def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache):
+    def stream_hint(self, norm):
+        return self.first_product_hint(norm, self.w_qkv)
+
+    def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
         fused = norm.fused_rmsnorm()
         if fused is None:
             return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache)
         qkv, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_qkv,
                                           self.ctx.dtype)
-        return self._attend(qkv, batch, cache, write_cache), resid
+        o = self._attend(qkv, batch, cache, write_cache)
+        return self.last_product(o, self.w_o, resid, hint), resid
 
     def forward(self, h, batch, cache, write_cache):
-        return self._attend(self.ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache,
-                            write_cache)
+        o = self._attend(self.ops.linear(h, self.w_qkv, self.ctx.dtype), batch, cache, write_cache)
+        return self.ops.linear(o, self.w_o, self.ctx.dtype)
 
     def _attend(self, qkv, batch, cache, write_cache):
         if cache is None:
@@ -107,4 +111,4 @@ class GroupedQueryAttention(Mixer):
             o = ops.paged_attention(q, batch, table, cache, num_heads=self.nq,
                                     num_kv_heads=self.nkv, head_dim=self.hd,
                                     scale=self.scale, window=self.window)
-        return ops.linear(o.view(T, self.nq * self.hd), self.w_o, self.ctx.dtype)
+        return o.view(T, self.nq * self.hd)

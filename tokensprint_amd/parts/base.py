@@ -18,6 +18,8 @@ from typing import Any, Callable
 
 import torch
 
+from tokensprint_amd.kernels.stream import NormHint
+
 
 # ------------------------------------------------------------------ declarations
 
@@ -79,6 +81,25 @@ class Part:
     def load(self, get: Callable[[str], torch.Tensor | None]) -> None:
         """Take the declared tensors (`get(name)`, None if optional and absent)."""
 
+    # -- the residual add and norm split over the product before and the product after
+    def first_product_hint(self, norm: "Norm", weight: torch.Tensor, silu_mul: bool = False):
+        """For `stream_hint` of a part whose first product is `weight` after `norm`: the
+        hint, if the norm is one a kernel may fuse and the provider has such kernels."""
+        fused = norm.fused_rmsnorm()
+        if fused is None or not hasattr(self.ops, "linear_into_stream"):
+            return None
+        return NormHint(fused[0], fused[1], weight, silu_mul)
+
+    def last_product(self, x: torch.Tensor, weight: torch.Tensor, resid: torch.Tensor, hint):
+        """The product that ends a sub-layer: x W^T as the stream's next delta, or, where
+        `hint` says what follows and the provider can, added into `resid` at once and
+        handed on as prepared rows (which stand in delta's place)."""
+        if hint is not None:
+            prepared = self.ops.linear_into_stream(x, weight, resid, hint)
+            if prepared is not None:
+                return prepared
+        return self.ops.linear(x, weight, self.ctx.dtype)
+
 
 class Norm(Part):
     def fused_rmsnorm(self):
@@ -118,10 +139,17 @@ class Mixer(Part):
         """h [T, width] -> [T, width].  `cache` is this run's cache view (or None)."""
         raise NotImplementedError
 
-    def forward_from_stream(self, resid, delta, norm: Norm, batch, cache, write_cache: bool):
+    def stream_hint(self, norm: Norm):
+        """A NormHint if this part, reading the stream through `norm`, takes prepared
+        rows in `delta`'s place (see `Part.last_product`), else None."""
+        return None
+
+    def forward_from_stream(self, resid, delta, norm: Norm, batch, cache, write_cache: bool,
+                            hint=None):
         """The same from the residual stream: adds `delta` (may be None) to `resid`,
         norms, mixes.  Returns (output, residual stream after the add).  A part overrides
-        this to fuse the add and the norm into its first product."""
+        this to fuse the add and the norm into its first product.  `hint` is the
+        `stream_hint` of whatever reads the stream next, or None; a part may ignore it."""
         h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
         return self.forward(h, batch, cache, write_cache), resid
 
@@ -130,7 +158,11 @@ class FeedForward(Part):
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
 
-    def forward_from_stream(self, resid, delta, norm: Norm, batch):
+    def stream_hint(self, norm: Norm):
+        """See Mixer.stream_hint."""
+        return None
+
+    def forward_from_stream(self, resid, delta, norm: Norm, batch, hint=None):
         """See Mixer.forward_from_stream."""
         h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
         return self.forward(h, batch), resid
@@ -141,7 +173,9 @@ class Block:
 
     The stream travels as (resid, delta): resid is float32 [T, width]; delta is
     the last sub-layer's output not yet added (None at the very start), so the
-    add can be fused into the next norm.
+    add can be fused into the next norm.  Where the part that reads the stream next
+    gives a `stream_hint`, the part before it may hand on prepared rows instead of a
+    delta (`Part.last_product`); only that reader ever sees them.
     """
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
@@ -153,7 +187,12 @@ class Block:
     def parts(self) -> list[Part]:
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward]
 
-    def forward(self, resid, delta, batch, cache, write_cache: bool):
+    def entry_hint(self):
+        """The `stream_hint` of the part of this block that reads the stream first."""
+        return None
+
+    def forward(self, resid, delta, batch, cache, write_cache: bool, next_hint=None):
+        """`next_hint`: the `entry_hint` of the block that runs next, or None."""
         raise NotImplementedError
 
 

@@ -34,13 +34,16 @@ class SwiGLU(FeedForward):
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = get(pre + "down_proj.weight")
 
-    def forward_from_stream(self, resid, delta, norm, batch):
+    def stream_hint(self, norm):
+        return self.first_product_hint(norm, self.w_gate_up, silu_mul=True)
+
+    def forward_from_stream(self, resid, delta, norm, batch, hint=None):
         fused = norm.fused_rmsnorm()
         if fused is None:
             return super().forward_from_stream(resid, delta, norm, batch)
         act, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_gate_up,
                                           self.ctx.dtype, silu_mul=True)
-        return self.ops.linear(act, self.w_down, self.ctx.dtype), resid
+        return self.last_product(act, self.w_down, resid, hint), resid
 
     def forward(self, h, batch):
         act = self.ops.linear_silu_mul(h, self.w_gate_up, self.ctx.dtype)
