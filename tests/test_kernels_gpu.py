@@ -514,6 +514,34 @@ def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
                                        rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("ctx", [700, 2500])
+def test_attend_finds_one_far_key_in_a_decode_step(ops, gpu_device, ctx):
+    """The same through the fused decode call (no norm, no rotation, so the query is the
+    row's own): one key at a page's, a block's or a split's edge dominates, or the step's
+    own key does, which is not in the cache when the walk starts."""
+    dtype = torch.bfloat16
+    nq, nkv, hd, page = 4, 2, 128, 16
+    kw = dict(num_heads=nq, num_kv_heads=nkv, kv_in_row=nkv, head_dim=hd, q_weight=None,
+              k_weight=None, eps=0.0, cos_sin=None, scale=1.0, window=None)
+    for far in (0, 15, 16, 31, 32, 127, 128, 255, 256, 511, 512, ctx - 2, ctx - 1, ctx):
+        batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                                spans=[(ctx, 1)], seed=23)
+        qkv = rand((1, (nq + 2 * nkv) * hd), dtype, gpu_device, 24)
+        row = qkv.view(nq + 2 * nkv, hd)
+        if far == ctx:       # the step's own key: 4 * q of the first head of its group
+            for kvh in range(nkv):
+                row[nq + kvh] = (4.0 * row[kvh * 2].float()).to(dtype)
+            want = [row[nq + nkv + kvh].float() for kvh in range(nkv)]
+        else:
+            phys = int(table[0, far // page])
+            for kvh in range(nkv):
+                cache.k_pages[phys, kvh, far % page] = (4.0 * row[kvh * 2].float()).to(dtype)
+            want = [cache.v_pages[phys, kvh, :, far % page].float() for kvh in range(nkv)]
+        out = ops.attend(qkv, batch, table, cache, True, **kw).view(1, nq, hd)
+        for kvh in range(nkv):
+            torch.testing.assert_close(out[0, kvh * 2].float(), want[kvh], rtol=2e-2, atol=2e-2)
+
+
 def test_argmax_and_ties(ops, gpu_device):
     logits = rand((9, 151936), torch.float32, gpu_device, 30)
     assert torch.equal(ops.argmax(logits).long(), logits.argmax(-1))
