@@ -147,9 +147,15 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
 }
 
 // Merge the splits of every tile: out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M),
-// splits taken in order.  One workgroup per item, thread (row, column group).
+// splits taken in order.  One workgroup per item, thread (row, column group).  A split
+// without keys has left m = -inf and is skipped.  Splits are taken eight at a time: the
+// loads of the eight, statistics and values, are all asked for before the first is used,
+// none under a condition, and the first eight do not wait for the position either (it
+// says how many splits hold keys at all, which ends the loop early when a short context
+// has been given many splits), so a merge of up to eight splits costs one trip to memory.
 template <int HD>
 __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs args) {
+  constexpr int kGroup = 8, DC = HD / 16;
   const AttentionArgs& a = args.base;
   const int item = blockIdx.x;
   const int tile = item / (a.nkv * args.head_blocks);
@@ -161,36 +167,52 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttentionMfmaArgs 
   const int r = threadIdx.x / 16, dc = threadIdx.x % 16;
   const int ti = r / args.rows_per_token, hh = hb * 16 + r % args.rows_per_token;
   if (ti >= ntok || hh >= group) return;
-  const int64_t base = (int64_t)item * args.num_splits * 16 + r;
+  const int S = args.num_splits;
+  const int64_t base = (int64_t)item * S * 16 + r;
   // splits beyond the tile's chunks hold nothing: same arithmetic as the first kernel
   const int pos_first = a.positions[tok0], pos_last = pos_first + ntok - 1;
-  const int lo_tile = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
-  const int nchunks = pos_last / kChunk - lo_tile / kChunk + 1;
-  const int per = (nchunks - 1 + args.num_splits) / args.num_splits;
-  const int used = min(args.num_splits, (nchunks + per - 1) / per);
-  // the loads of a split's statistics and of its values do not wait for one another
-  float M = -INFINITY;
-  for (int s = 0; s < used; ++s)
-    M = fmaxf(M, args.partial_ml[(base + (int64_t)s * 16) * 2]);
-  float L = 0.f;
-  float acc[HD / 16] = {};
-  for (int s = 0; s < used; ++s) {
-    const int64_t slot = base + (int64_t)s * 16;
-    const float ms = args.partial_ml[slot * 2];
-    const float ls = args.partial_ml[slot * 2 + 1];
-    float part[HD / 16];
+  float M = -INFINITY, L = 0.f;
+  float acc[DC] = {};
+  int used = S;                              // known after the first group's loads
+  for (int s0 = 0; s0 < used; s0 += kGroup) {
+    float ms[kGroup], ls[kGroup], part[kGroup][DC];
 #pragma unroll
-    for (int i = 0; i < HD / 16; ++i) part[i] = args.partial_o[slot * HD + i * 16 + dc];
-    if (ms == -INFINITY) continue;       // an empty split wrote no values: ignore what is there
-    const float w = __builtin_amdgcn_exp2f(ms - M);
-    L += ls * w;
+    for (int j = 0; j < kGroup; ++j) {
+      const int64_t slot = base + (int64_t)min(s0 + j, S - 1) * 16;   // past the end: the last again
+      ms[j] = args.partial_ml[slot * 2];
+      ls[j] = args.partial_ml[slot * 2 + 1];
 #pragma unroll
-    for (int i = 0; i < HD / 16; ++i) acc[i] += part[i] * w;
+      for (int i = 0; i < DC; ++i) part[j][i] = args.partial_o[slot * HD + i * 16 + dc];
+    }
+    if (s0 == 0) {
+      const int lo_tile = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+      const int nchunks = pos_last / kChunk - lo_tile / kChunk + 1;
+      const int per = (nchunks - 1 + S) / S;
+      used = min(S, (nchunks + per - 1) / per);
+    }
+    float Mg = M;
+#pragma unroll
+    for (int j = 0; j < kGroup; ++j) Mg = (s0 + j < S) ? fmaxf(Mg, ms[j]) : Mg;
+    if (Mg == -INFINITY) continue;            // nothing but empty splits so far
+    const float keep = __builtin_amdgcn_exp2f(M - Mg);     // M = -inf gives 0
+    L *= keep;
+#pragma unroll
+    for (int i = 0; i < DC; ++i) acc[i] *= keep;
+#pragma unroll
+    for (int j = 0; j < kGroup; ++j) {
+      // an empty split wrote no values: what is there is dropped, not multiplied by 0
+      const bool live = s0 + j < S && ms[j] != -INFINITY;
+      const float w = live ? __builtin_amdgcn_exp2f(ms[j] - Mg) : 0.f;
+      L += live ? ls[j] * w : 0.f;
+#pragma unroll
+      for (int i = 0; i < DC; ++i) acc[i] += live ? part[j][i] * w : 0.f;
+    }
+    M = Mg;
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;
   bf16_t* out = (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + kvh * group + hh) * HD;
 #pragma unroll
-  for (int i = 0; i < HD / 16; ++i) out[i * 16 + dc] = (bf16_t)(acc[i] * inv);
+  for (int i = 0; i < DC; ++i) out[i * 16 + dc] = (bf16_t)(acc[i] * inv);
 }
 
 int ts_check_attention_args(const AttentionArgs& a, const char* who);
