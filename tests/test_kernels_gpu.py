@@ -514,6 +514,48 @@ def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
                                        rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("nq,nkv,hd,page,window", [(16, 8, 128, 16, None), (16, 8, 128, 64, 700),
+                                                   (8, 8, 96, 16, None), (6, 2, 64, 32, None),
+                                                   (40, 2, 32, 16, 300)])
+def test_attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
+    """Portions of prompts long enough for the kernels in which a wavefront walks several
+    query tiles: with and without norm weights, rotation, and keys in the row; groups of
+    3 and 20 heads, whose 16 rows are not a whole number of tokens (a row past a tile's
+    tokens must not be computed with that tile's key range and stored)."""
+    dtype = torch.bfloat16
+    group = nq // nkv
+    per_tile = 16 // min(group, 16)
+    need = -(-2048 // (nkv * -(-group // 16))) * per_tile          # tokens for 2048 wave tiles
+    spans = [(0, need // 2 + 37), (300, need // 2 + 100), (17, 150)]
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=71)
+    tiles16 = sum(-(-n // per_tile) for _, n in spans)
+    assert tiles16 * nkv * -(-group // 16) >= 2048
+    T = batch.num_tokens
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 73)
+    wk = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 74)
+    angles = torch.outer(torch.arange(batch.max_ctx_len + 8, dtype=torch.float32),
+                         1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    variants = [(nkv, True, True), (0, True, True)]
+    if (nq, hd) == (16, 128):
+        variants += [(nkv, False, True), (nkv, True, False)]
+    for kv_in_row, norm, rot in variants:
+        qkv = rand((T, (nq + 2 * kv_in_row) * hd), dtype, gpu_device, 72)
+        mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                           cache.k_pages.clone(), cache.v_pages.clone())
+        theirs = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                             cache.k_pages.clone(), cache.v_pages.clone())
+        kw = dict(num_heads=nq, num_kv_heads=nkv, kv_in_row=kv_in_row, head_dim=hd,
+                  q_weight=wq if norm else None, k_weight=wk if norm else None, eps=1e-6,
+                  cos_sin=cos_sin if rot else None, scale=hd ** -0.5, window=window)
+        out = ops.attend(qkv, batch, table, mine, bool(kv_in_row), **kw)
+        ref = REF.attend(qkv, batch, table, theirs, bool(kv_in_row), **kw)
+        torch.testing.assert_close(mine.k_pages.float(), theirs.k_pages.float(), **tol(dtype))
+        torch.testing.assert_close(mine.v_pages.float(), theirs.v_pages.float(), **tol(dtype))
+        torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
 @pytest.mark.parametrize("ctx", [700, 2500])
 def test_attend_finds_one_far_key_in_a_decode_step(ops, gpu_device, ctx):
     """The same through the fused decode call (no norm, no rotation, so the query is the

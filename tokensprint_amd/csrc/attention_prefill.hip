@@ -42,7 +42,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
 #pragma unroll
   for (int j = 0; j < TPW; ++j) {
     const int t = j * tq + ti;
-    const bool row_ok = t < ntok && hh < group;
+    // (16 rows need not be a whole number of tokens: a row past the tile's tokens would
+    // be the next tile's token with this tile's key range, stored over the right result)
+    const bool row_ok = ti < tq && t < ntok && hh < group;
     ts[j].pos = row_ok ? pos_first + t : -1;
     ts[j].lo = (a.window > 0) ? max(0, ts[j].pos - a.window + 1) : 0;
     tile_first[j] = pos_first + j * tq;
@@ -127,7 +129,9 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   const int ti = wave * tq + r / args.rows_per_token;
   const int hh = hb * 16 + r % args.rows_per_token;
   const int head = kvh * group + min(hh, group - 1);
-  const bool row_ok = ti < ntok && hh < group;
+  // (16 rows need not be a whole number of tokens: a row past the tile's tokens would be
+  // the next wave's token with this wave's key range, stored over the right result)
+  const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
   const int pos_first = uniform(a.positions[tok0]);
   const int pos_last = pos_first + ntok - 1;
   const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
