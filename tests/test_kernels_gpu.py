@@ -381,18 +381,33 @@ def test_paged_attention_long_contexts(ops, gpu_device, dtype, window):
 
 @pytest.mark.parametrize("window", [None, 100])
 @pytest.mark.parametrize("nq,nkv,hd,page", [(16, 8, 128, 16), (8, 2, 64, 16), (6, 3, 48, 8),
-                                            (4, 4, 256, 32), (32, 1, 32, 16)])
+                                            (4, 4, 256, 32), (32, 1, 32, 16), (6, 2, 64, 32),
+                                            (10, 2, 32, 12), (40, 2, 32, 16), (3, 1, 128, 64)])
 def test_paged_attention_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
-    """Portions long enough for the multi-tile prompt kernel (bfloat16), with and without
-    cached context before them, beside a decode token."""
+    """Portions long enough for the kernels in which a wavefront walks several query tiles
+    (bfloat16; pages that are powers of two share blocks through LDS, others do not),
+    with and without cached context before them, beside a decode token.  Groups of 3, 5
+    and 20 heads: 16 rows are then not a whole number of tokens."""
     dtype = torch.bfloat16
-    spans = [(0, 700), (333, 1), (50, 515)]
+    group = nq // nkv
+    per_tile = 16 // min(group, 16)
+    need = -(-2048 // (nkv * -(-group // 16))) * per_tile          # tokens for 2048 wave tiles
+    spans = [(0, need // 2 + 188), (333, 1), (50, need // 2 + 3)]
     batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
                                             spans=spans, seed=33)
+    assert ops._prefill_tiles(batch, nkv, group) is not None
     q = rand((batch.num_tokens, nq, hd), dtype, gpu_device, 34)
     kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
     out = ops.paged_attention(q, batch, table, cache, **kw)
-    pick = [0, 1, 7, 8, 15, 16, 31, 32, 33, 255, 256, 699, 700, 701, 702, 709, 900, 1215]
+    T, first = batch.num_tokens, spans[0][1]
+    if T <= 3000:
+        pick = list(range(T))
+    else:       # the first tokens, both portions' ends and starts, and tile borders all over
+        step = 4 * per_tile
+        pick = sorted(set(list(range(0, 70)) + list(range(first - 40, first + 70)) +
+                          list(range(T - 70, T)) +
+                          [t + d for t in range(step * 7, T - step, step * 29)
+                           for d in (-1, 0, 1, per_tile - 1, per_tile)]))
     import copy
     sub = copy.copy(batch)
     sub.positions = batch.positions[pick].contiguous()

@@ -551,8 +551,7 @@ class HipOps:
         m.base = a
         m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
         # long portions of prompts: a wavefront takes several query tiles and walks alone
-        tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
-        if tiles16 * a.nkv * head_blocks >= 2048:
+        if self._prefill_tiles(batch, a.nkv, group) is not None:
             tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size)
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
@@ -581,6 +580,13 @@ class HipOps:
             pml = torch.empty(items * splits * 16 * 2, dtype=torch.float32, device=self.device)
             m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
         self._call(self.lib.ts_attention_mfma, byref(m), self._stream())
+
+    def _prefill_tiles(self, batch, num_kv_heads, group):
+        """Tokens per 16-row tile if the step is one of long portions of prompts (enough
+        tiles to fill the chip with wavefronts that walk alone), else None."""
+        tokens_per_tile = 16 // min(group, 16)
+        tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
+        return tokens_per_tile if tiles16 * num_kv_heads * -(-group // 16) >= 2048 else None
 
     def _attention_tiles(self, batch, tokens):
         """Device list of (entry, first flat token, tokens) cutting every entry of the batch
