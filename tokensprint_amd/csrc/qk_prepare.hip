@@ -106,7 +106,12 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_qk;
 typedef __attribute__((ext_vector_type(4))) float f32x4_qk;
 
-template <typename TC>
+// A thread goes through its piece (N of them: one was measured best, more waves do
+// better than longer ones) in three rounds: everything that hangs on nothing (the
+// elements, the position, the norm weight, the entry), then what hangs on the position
+// (cos and sin, the page), then the arithmetic and the stores.  A piece so costs two
+// trips to memory, not one per use.
+template <typename TC, int N>
 __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, int lanes_log2,
                                                              int with_v) {
   const int L = 1 << lanes_log2;                     // lanes per head
@@ -115,80 +120,109 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, in
   const int sub = lane & (L - 1);                    // my 8 elements: [8*sub, 8*sub + 8)
   const int heads = a.nq + (a.store_kv ? (with_v ? 2 : 1) * a.nkv : 0);
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  const int64_t item = wave * heads_per_wave + (lane >> lanes_log2);
-  const bool live = item < (int64_t)a.num_tokens * heads;
-  const int64_t it = live ? item : 0;
-  const int t = (int)(it / heads), h = (int)(it % heads);
   const int hd = a.hd, half = hd / 2;
-  const int pos = a.positions[t];
-  const int kind = h < a.nq ? 0 : (h < a.nq + a.nkv ? 1 : 2);
-  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * (a.nq + 2 * a.nkv) * hd + (int64_t)h * hd;
-  const bf16x8_qk x = *(const bf16x8_qk*)(src + sub * 8);
-  float v[8];
+  const f32x4_qk zero4 = {0.f, 0.f, 0.f, 0.f};
+  const int i0 = (sub & (L / 2 - 1)) * 8;            // index into the half-size table
+  struct Piece {
+    bool live, norm, rotate, to_page;
+    int t, h, kind, pos, entry, page;
+    bf16x8_qk x;
+    f32x4_qk w0, w1, c0, c1, s0, s1;
+  };
+  Piece pc[N];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = (float)x[j];
-
-  const float* w = kind == 0 ? a.q_weight : a.k_weight;
-  if (kind != 2 && w) {
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
-    for (int o = 1; o < L; o <<= 1) ss += __shfl_xor(ss, o, kWave);
-    const float rstd = rsqrtf(ss / (float)hd + a.eps);
-    const f32x4_qk w0 = *(const f32x4_qk*)(w + sub * 8), w1 = *(const f32x4_qk*)(w + sub * 8 + 4);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { v[j] *= rstd * w0[j]; v[4 + j] *= rstd * w1[j]; }
-  }
-  if (kind != 2 && a.cos) {
-    const bool first = sub < L / 2;                  // holds elements i < hd/2
-    const int i0 = (sub & (L / 2 - 1)) * 8;          // index into the half-size table
-    const f32x4_qk c0 = *(const f32x4_qk*)(a.cos + (int64_t)pos * half + i0),
-                   c1 = *(const f32x4_qk*)(a.cos + (int64_t)pos * half + i0 + 4),
-                   s0 = *(const f32x4_qk*)(a.sin + (int64_t)pos * half + i0),
-                   s1 = *(const f32x4_qk*)(a.sin + (int64_t)pos * half + i0 + 4);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float other = __shfl_xor(v[j], L / 2, kWave);
-      const float c = j < 4 ? c0[j] : c1[j - 4], sn = j < 4 ? s0[j] : s1[j - 4];
-      // first half: re*c - im*s with im = other; second half: im*c + re*s with re = other
-      v[j] = first ? v[j] * c - other * sn : v[j] * c + other * sn;
+  for (int i = 0; i < N; ++i) {
+    Piece& p = pc[i];
+    const int64_t item = (wave * N + i) * heads_per_wave + (lane >> lanes_log2);
+    p.live = item < (int64_t)a.num_tokens * heads;
+    const int64_t it = p.live ? item : 0;
+    p.t = (int)(it / heads), p.h = (int)(it % heads);
+    p.kind = p.h < a.nq ? 0 : (p.h < a.nq + a.nkv ? 1 : 2);
+    const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)p.t * (a.nq + 2 * a.nkv) * hd + (int64_t)p.h * hd;
+    p.x = *(const bf16x8_qk*)(src + sub * 8);
+    p.pos = a.positions[p.t];
+    const float* w = p.kind == 0 ? a.q_weight : a.k_weight;
+    p.norm = p.kind != 2 && w, p.rotate = p.kind != 2 && a.cos;
+    p.to_page = p.kind != 0 && a.paged;
+    p.w0 = p.w1 = zero4;
+    if (p.norm) {
+      p.w0 = *(const f32x4_qk*)(w + sub * 8);
+      p.w1 = *(const f32x4_qk*)(w + sub * 8 + 4);
     }
+    p.entry = p.to_page ? a.entry_of_token[p.t] : 0;
   }
-  if (!live) return;
-
-  if (kind == 0) {
-    bf16x8_qk o;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = (bf16_t)v[j];
-    *(bf16x8_qk*)((bf16_t*)a.q_out + ((int64_t)t * a.nq + h) * hd + sub * 8) = o;
-    return;
+  for (int i = 0; i < N; ++i) {
+    Piece& p = pc[i];
+    p.c0 = p.c1 = p.s0 = p.s1 = zero4;
+    if (p.rotate) {
+      const float* cp = a.cos + (int64_t)p.pos * half + i0;
+      const float* sp = a.sin + (int64_t)p.pos * half + i0;
+      p.c0 = *(const f32x4_qk*)cp; p.c1 = *(const f32x4_qk*)(cp + 4);
+      p.s0 = *(const f32x4_qk*)sp; p.s1 = *(const f32x4_qk*)(sp + 4);
+    }
+    p.page = p.to_page ? a.table[(int64_t)p.entry * a.table_width + p.pos / a.page_size] : -1;
   }
-  const int kvh = kind == 1 ? h - a.nq : h - a.nq - a.nkv;
-  if (!a.paged) {
-    TC* dst = (TC*)(kind == 1 ? a.k_dst : a.v_dst) + ((int64_t)t * a.nkv + kvh) * hd + sub * 8;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dst[j] = from_f32<TC>(v[j]);
-    return;
-  }
-  const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
-  if (page < 0) return;
-  const int64_t head_base = ((int64_t)page * a.nkv + kvh) * a.page_size * hd;
-  const int slot = pos % a.page_size;
-  if (kind == 1) {
-    TC* dst = (TC*)a.k_dst + head_base + (int64_t)slot * hd + sub * 8;
-    if constexpr (sizeof(TC) == 2) {     // one 16-byte store (pages and rows are 16-byte aligned)
+  for (int i = 0; i < N; ++i) {
+    const Piece& p = pc[i];
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (float)p.x[j];
+    if (p.norm) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+      for (int o = 1; o < L; o <<= 1) ss += __shfl_xor(ss, o, kWave);
+      const float rstd = rsqrtf(ss / (float)hd + a.eps);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { v[j] *= rstd * p.w0[j]; v[4 + j] *= rstd * p.w1[j]; }
+    }
+    if (p.rotate) {
+      const bool first = sub < L / 2;                  // holds elements i < hd/2
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float other = __shfl_xor(v[j], L / 2, kWave);
+        const float c = j < 4 ? p.c0[j] : p.c1[j - 4], sn = j < 4 ? p.s0[j] : p.s1[j - 4];
+        // first half: re*c - im*s with im = other; second half: im*c + re*s with re = other
+        v[j] = first ? v[j] * c - other * sn : v[j] * c + other * sn;
+      }
+    }
+    if (!p.live) continue;
+    const int t = p.t, h = p.h;
+    if (p.kind == 0) {
       bf16x8_qk o;
 #pragma unroll
       for (int j = 0; j < 8; ++j) o[j] = (bf16_t)v[j];
-      *(bf16x8_qk*)dst = o;
-    } else {
+      *(bf16x8_qk*)((bf16_t*)a.q_out + ((int64_t)t * a.nq + h) * hd + sub * 8) = o;
+      continue;
+    }
+    const int kvh = p.kind == 1 ? h - a.nq : h - a.nq - a.nkv;
+    if (!a.paged) {
+      TC* dst = (TC*)(p.kind == 1 ? a.k_dst : a.v_dst) + ((int64_t)t * a.nkv + kvh) * hd + sub * 8;
 #pragma unroll
       for (int j = 0; j < 8; ++j) dst[j] = from_f32<TC>(v[j]);
+      continue;
     }
-  } else {
-    TC* dst = (TC*)a.v_dst + head_base + slot;
+    if (p.page < 0) continue;
+    const int64_t head_base = ((int64_t)p.page * a.nkv + kvh) * a.page_size * hd;
+    const int slot = p.pos % a.page_size;
+    if (p.kind == 1) {
+      TC* dst = (TC*)a.k_dst + head_base + (int64_t)slot * hd + sub * 8;
+      if constexpr (sizeof(TC) == 2) {     // one 16-byte store (pages and rows are 16-byte aligned)
+        bf16x8_qk o;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dst[(int64_t)(sub * 8 + j) * a.page_size] = from_f32<TC>(v[j]);
+        for (int j = 0; j < 8; ++j) o[j] = (bf16_t)v[j];
+        *(bf16x8_qk*)dst = o;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = from_f32<TC>(v[j]);
+      }
+    } else {
+      TC* dst = (TC*)a.v_dst + head_base + slot;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[(int64_t)(sub * 8 + j) * a.page_size] = from_f32<TC>(v[j]);
+    }
   }
 }
 
@@ -244,7 +278,7 @@ extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_
     const int64_t vblocks = (vec_items + heads_per_block - 1) / heads_per_block;
     if (vblocks > 2147483647LL) TS_FAIL("qk_prepare: too many tokens");
     TS_DISPATCH_TYPE(cache_type, TC,
-        hipLaunchKernelGGL((qk_prepare_vec_kernel<TC>), dim3((unsigned)vblocks),
+        hipLaunchKernelGGL((qk_prepare_vec_kernel<TC, 1>), dim3((unsigned)vblocks),
                            dim3(waves_per_block * kWave), 0, stream, a, lanes_log2,
                            v_tiles ? 0 : 1));
     if (v_tiles)
