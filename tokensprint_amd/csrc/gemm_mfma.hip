@@ -464,8 +464,10 @@ extern "C" int ts_norm_gemm_mfma_bf16(const float* resid_in, const void* delta, 
 //
 // ts_gemm_tail_bf16: resid[M, N] += bf16(A[M, K] W[N, K]^T) in place (float32), and for
 // the RMSNorm with weight norm_w that follows: prepared[M, N] = bf16(resid * norm_w) and
-// sumsq[ceil(N / 16)][M], each row's sum of squares of resid over 16 columns.
+// sumsq[ts_gemm_tail_parts(M, N)][M], each row's sum of squares of resid over a slice of
+// its columns (16, or fewer where the product is spread over more workgroups).
 extern "C" int ts_gemm_tail_fits(int M, int N, int K) { return gemm_direct_tail_fits(M, N, K); }
+extern "C" int ts_gemm_tail_parts(int M, int N) { return gemm_direct_tail_parts(M, N); }
 
 extern "C" int ts_gemm_tail_bf16(const void* a, const void* w, float* resid, const float* norm_w,
                                  void* prepared, float* sumsq, int M, int N, int K,
@@ -486,22 +488,22 @@ extern "C" int ts_gemm_tail_bf16(const void* a, const void* w, float* resid, con
 }
 
 // ts_gemm_scaled_bf16: C[M, N] = (prepared[M, K] W[N, K]^T) * rsqrt(sum_j sumsq[j][m] / K + eps)
-// for sumsq[ceil(K / 16)][M]; pair as in ts_gemm_mfma_bf16.
-extern "C" int ts_gemm_scaled_fits(int M, int N, int K, int pair) {
-  return gemm_direct_scaled_fits(M, N, K, pair != 0);
+// for sumsq[parts][M]; pair as in ts_gemm_mfma_bf16.
+extern "C" int ts_gemm_scaled_fits(int M, int N, int K, int pair, int parts) {
+  return gemm_direct_scaled_fits(M, N, K, pair != 0, parts);
 }
 
-extern "C" int ts_gemm_scaled_bf16(const void* prepared, const float* sumsq, float eps,
+extern "C" int ts_gemm_scaled_bf16(const void* prepared, const float* sumsq, int parts, float eps,
                                    const void* w, void* c, int c_type, int M, int N, int K,
                                    int pair, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (!gemm_direct_scaled_fits(M, N, K, pair != 0))
+  if (!gemm_direct_scaled_fits(M, N, K, pair != 0, parts))
     TS_FAIL("gemm_scaled: M=%d, N=%d, K=%d is not a product the scaled form takes", M, N, K);
   if (((uintptr_t)prepared | (uintptr_t)w) & 15) TS_FAIL("gemm_scaled: operands must be 16-byte aligned");
   if (!prepared || !sumsq || !w || !c) TS_FAIL("gemm_scaled: null operand");
   DirectArgs da = {};
   da.A = (const bf16_t*)prepared; da.W = (const bf16_t*)w; da.C = c; da.M = M; da.N = N; da.K = K;
-  da.sumsq = sumsq; da.parts = (K + 15) / 16; da.eps = eps;
+  da.sumsq = sumsq; da.parts = parts; da.eps = eps;
   if (gemm_direct_launch(da, c_type, pair != 0, false, stream)) return -1;
   TS_CHECK_LAUNCH("gemm_scaled");
   return 0;

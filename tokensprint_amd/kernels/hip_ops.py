@@ -246,15 +246,16 @@ class HipOps:
         if weight.shape[1] != K:
             raise ValueError(f"linear_into_stream: x has {K} columns, weight has {weight.shape[1]}")
         next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
+        parts = self.lib.ts_gemm_tail_parts(M, N)
         if hint.weight.shape[1] != N or self._library_rows(M, N, K) \
                 or self._library_rows(M, next_n, N) \
                 or self.lib.ts_gemm_tail_fits(M, N, K) != 1 \
-                or self.lib.ts_gemm_scaled_fits(M, next_n, N, int(hint.silu_mul)) != 1:
+                or self.lib.ts_gemm_scaled_fits(M, next_n, N, int(hint.silu_mul), parts) != 1:
             return None
         self._check("resid", resid, torch.float32, shape=(M, N))
         self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
         rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
-        sumsq = torch.empty((N + 15) // 16, M, dtype=torch.float32, device=self.device)
+        sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_gemm_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
                    _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, self._stream())
         return PreparedRows(rows, sumsq, hint)
@@ -272,7 +273,7 @@ class HipOps:
             raise ValueError(f"norm_linear: prepared rows cannot give {out_dtype}")
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         self._call(self.lib.ts_gemm_scaled_bf16, _ptr(prepared.rows), _ptr(prepared.sumsq),
-                   c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                   prepared.sumsq.shape[0], c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
                    int(silu_mul), self._stream())
         return out, resid
 
