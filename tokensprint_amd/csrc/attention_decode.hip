@@ -74,7 +74,11 @@ __device__ __forceinline__ void prepare_head(bf16x8 (&v)[HD / 32], bool live, bo
     if (rotate) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float other = __shfl_xor(x[j], 32, kWave);
+        // the partner's element, from the lane 32 further: a row-swap instruction, fed
+        // the same value twice, returns each half's value in both halves
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x[j]), __float_as_uint(x[j]),
+                                                         false, false);
+        const float other = __uint_as_float(first ? sw[1] : sw[0]);
         const float c = cs[s][j / 4][j % 4], sn = cs[s][2 + j / 4][j % 4];
         x[j] = first ? x[j] * c - other * sn : x[j] * c + other * sn;
       }
@@ -125,11 +129,12 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     return;
   }
 
-  // fused form: the last wave does not walk; it prepares the query rows for the others
-  // and, in the first split, takes the new key
+  // fused form: the last wave does not walk; it prepares the query rows for the others.
+  // In the first split the wave before it does not walk either: it takes the new key,
+  // side by side with the last wave's work on the queries.
   const bool prep_wave = FUSED && wave == NW - 1;
-  const bool key_wave = adds_new && prep_wave;
-  const int walkers = FUSED ? NW - 1 : NW;
+  const bool key_wave = adds_new && wave == NW - 2;
+  const int walkers = FUSED ? NW - 1 - (adds_new ? 1 : 0) : NW;
 
   TileState<HD> t;
   t.pos = row_ok ? last : -1;
@@ -137,7 +142,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   const float scale_log2 = a.scale * 1.44269504088896341f;
   const int stride = walkers * 32;
   const int key_begin = max(c0 * kChunk, lo & ~31) + wave * 32;
-  const int key_end = prep_wave ? 0 : min(c1 * kChunk, last + 1);
+  const int key_end = (prep_wave || key_wave) ? 0 : min(c1 * kChunk, last + 1);
   PageCursor cur{(ConstTable)table, a.page_size, last, -1, -1};
   KvBlock<HD> A, B;
 
@@ -149,51 +154,43 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     const int row_width = (a.nq + 2 * args.kv_in_row) * HD;
     const bf16_t* row = args.qkv + (int64_t)token * row_width;
     const bool rotate = args.cos != nullptr;
-    if (!prep_wave) {
+    const bool walker = !prep_wave && !key_wave;
+    if (walker) {
       cur.start(key_begin);
       if (key_begin < key_end) load_kv_block<HD, true>(A, a, table, cur, kvh, key_begin, stride, r, g);
     }
-    f32x4 cs[KS][4];          // cos (2 x 4) and sin (2 x 4) of the lane's elements
-    f32x4 qw[KS][2], kw[KS][2];
+    // the head vector a wave that does not walk prepares: the query rows, or the new key
+    // (the same in all 16 rows)
     bf16x8 kq[KS];
-    if (prep_wave) {
-      if (rotate) {
+    if (!walker) {
+      const float* weight = prep_wave ? args.q_weight : args.k_weight;
+      const bf16_t* src = row + (int64_t)(prep_wave ? head : a.nq + kvh) * HD + g * (HD / 4);
+      f32x4 cs[KS][4];          // cos (2 x 4) and sin (2 x 4) of the lane's elements
+      f32x4 w[KS][2];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
+      for (int s = 0; s < KS; ++s) {
+        kq[s] = *(const bf16x8*)(src + s * 8);
+        if (rotate) {
           const int64_t i = (int64_t)pos * (HD / 2) + (g & 1) * (HD / 4) + s * 8;
           cs[s][0] = *(const f32x4*)(args.cos + i);
           cs[s][1] = *(const f32x4*)(args.cos + i + 4);
           cs[s][2] = *(const f32x4*)(args.sin + i);
           cs[s][3] = *(const f32x4*)(args.sin + i + 4);
         }
-      }
-      auto load_weight = [&](const float* weight, f32x4 (&w)[KS][2]) {
-        if (!weight) return;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
+        if (weight) {
           w[s][0] = *(const f32x4*)(weight + g * (HD / 4) + s * 8);
           w[s][1] = *(const f32x4*)(weight + g * (HD / 4) + s * 8 + 4);
         }
-      };
-      load_weight(args.q_weight, qw);
-      const bf16_t* qrow = row + (int64_t)head * HD + g * (HD / 4);
-#pragma unroll
-      for (int s = 0; s < KS; ++s) t.q[s] = *(const bf16x8*)(qrow + s * 8);
-      if (key_wave) {
-        load_weight(args.k_weight, kw);
-        const bf16_t* krow = row + (int64_t)(a.nq + kvh) * HD + g * (HD / 4);
-#pragma unroll
-        for (int s = 0; s < KS; ++s) kq[s] = *(const bf16x8*)(krow + s * 8);
       }
-      prepare_head<HD>(t.q, row_ok, args.q_weight != nullptr, qw, args.eps, cs, rotate, g);
+      prepare_head<HD>(kq, prep_wave ? row_ok : true, weight != nullptr, w, args.eps, cs, rotate, g);
+      if (prep_wave) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) s_q[s][lane] = t.q[s];
+        for (int s = 0; s < KS; ++s) s_q[s][lane] = kq[s];
+      }
     }
     __syncthreads();
-    if (!prep_wave) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) t.q[s] = s_q[s][lane];
-    }
+    for (int s = 0; s < KS; ++s) t.q[s] = s_q[s][lane];
 #pragma unroll
     for (int db = 0; db < DB; ++db) t.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
     t.m = -INFINITY;
@@ -201,7 +198,6 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
 
     if (key_wave) {
       const bf16_t* vrow = row + (int64_t)(a.nq + args.kv_in_row + kvh) * HD;
-      prepare_head<HD>(kq, true, args.k_weight != nullptr, kw, args.eps, cs, rotate, g);
       float dot = 0.f;
 #pragma unroll
       for (int s = 0; s < KS; ++s)
