@@ -251,58 +251,58 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   f32x4 (&o)[DB] = t.o;
   float m = t.m, l = row_sum<HD>(t);
 
-  // the waves' partial results (the new key's among them), merged by wave 0 in wave order
-  __shared__ float s_ml[NW - 1][kWave][2];
-  __shared__ f32x4 s_o[NW - 1][DB][kWave];
-  if (wave > 0) {
-    s_ml[wave - 1][lane][0] = m;
-    s_ml[wave - 1][lane][1] = l;
+  // The waves' partial results (the new key's among them) all go to LDS, and every wave
+  // merges, in wave order, its share of the head's blocks of 16 elements and stores that
+  // share: the merge is as wide as the workgroup instead of one wave's long tail.
+  extern __shared__ __attribute__((aligned(16))) unsigned char merge_lds[];
+  float (*s_ml)[kWave][2] = (float (*)[kWave][2])merge_lds;                        // [NW]
+  f32x4 (*s_o)[DB][kWave] = (f32x4 (*)[DB][kWave])(merge_lds + NW * kWave * 2 * 4);  // [NW]
+  s_ml[wave][lane][0] = m;
+  s_ml[wave][lane][1] = l;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) s_o[wave - 1][db][lane] = o[db];
-  }
+  for (int db = 0; db < DB; ++db) s_o[wave][db][lane] = o[db];
   __syncthreads();
-  if (wave > 0) return;
-  float M = m;
+  constexpr int kShare = (DB + NW - 1) / NW;         // blocks of 16 elements per wave
+  if (wave * kShare >= DB) return;
+  float M = -INFINITY;
 #pragma unroll
-  for (int w = 0; w < NW - 1; ++w) M = fmaxf(M, s_ml[w][lane][0]);
-  if (M != -INFINITY) {
-    const float w0 = __builtin_amdgcn_exp2f(m - M);     // m = -inf gives 0
-    l *= w0;
+  for (int w = 0; w < NW; ++w) M = fmaxf(M, s_ml[w][lane][0]);
+  float ww[NW];
+  l = 0.f;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) o[db][i] *= w0;
-#pragma unroll
-    for (int w = 0; w < NW - 1; ++w) {
-      const float mw = s_ml[w][lane][0];
-      if (mw == -INFINITY) continue;
-      const float ww = __builtin_amdgcn_exp2f(mw - M);
-      l += s_ml[w][lane][1] * ww;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const f32x4 ow = s_o[w][db][lane];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[db][i] += ow[i] * ww;
-      }
-    }
-    m = M;
+  for (int w = 0; w < NW; ++w) {
+    const float mw = s_ml[w][lane][0];
+    // a wave that saw no key has m = -inf (and so has everyone if M is): weight 0
+    ww[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+    l += s_ml[w][lane][1] * ww[w];
   }
-
+  m = M;
   // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
-  if (ma.num_splits == 1) {
-    if (!row_ok) return;
-    store_tile<HD>(t, l, (bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD, g);
-  } else {
-    const int64_t slot = ((int64_t)item * ma.num_splits + split) * 16 + r;
-    if (row_ok) {
-      float* po = ma.partial_o + slot * HD;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const int64_t slot = ((int64_t)item * ma.num_splits + split) * 16 + r;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) *(f32x4*)(po + db * 16 + g * 4) = o[db];
+  for (int k = 0; k < kShare; ++k) {
+    const int db = wave * kShare + k;
+    if (db >= DB) break;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const f32x4 ow = s_o[w][db][lane];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += ww[w] == 0.f ? 0.f : ow[i] * ww[w];   // never 0 * garbage
     }
-    if (g == 0) {
-      ma.partial_ml[slot * 2] = m;
-      ma.partial_ml[slot * 2 + 1] = l;
+    if (!row_ok) continue;
+    if (ma.num_splits == 1) {
+      bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv),
+                   (bf16_t)(acc[3] * inv)};
+      *(bf16x4*)((bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD + db * 16 + g * 4) = ov;
+    } else {
+      *(f32x4*)(ma.partial_o + slot * HD + db * 16 + g * 4) = acc;
     }
+  }
+  if (ma.num_splits > 1 && wave == 0 && g == 0) {
+    ma.partial_ml[slot * 2] = m;
+    ma.partial_ml[slot * 2 + 1] = l;
   }
 }
 
@@ -313,13 +313,32 @@ static int launch_decode(const AttentionDecodeArgs& args, hipStream_t stream) {
   const AttentionMfmaArgs& m = args.m;
   const int items = m.num_tiles * m.base.nkv * m.head_blocks;
   const dim3 grid(items, m.num_splits), block(decode_waves<HD>() * kWave);
+  // the merge area: per wave its row statistics and HD/16 blocks of partial sums
+  const size_t lds = (size_t)decode_waves<HD>() * (kWave * 2 * 4 + (HD / 16) * kWave * 16);
   if (args.qkv) {
-    if constexpr (HD % 32 == 0)
-      hipLaunchKernelGGL((attention_decode_kernel<HD, true>), grid, block, 0, stream, args);
-    else
+    if constexpr (HD % 32 == 0) {
+      auto kernel = attention_decode_kernel<HD, true>;
+      static bool raised = false;     // per head size
+      if (lds > 48 * 1024 && !raised) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+          TS_FAIL("attention_decode: cannot raise the LDS limit to %zu bytes", lds);
+        raised = true;
+      }
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
+    } else {
       TS_FAIL("attention_decode: the fused form needs a head size that is a multiple of 32");
+    }
   } else {
-    hipLaunchKernelGGL((attention_decode_kernel<HD, false>), grid, block, 0, stream, args);
+    auto kernel = attention_decode_kernel<HD, false>;
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
+      if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess)
+        TS_FAIL("attention_decode: cannot raise the LDS limit to %zu bytes", lds);
+      raised = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
   }
   if (m.num_splits > 1) return launch_attention_merge(m, stream);
   return 0;
