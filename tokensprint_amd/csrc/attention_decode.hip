@@ -110,12 +110,51 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   const int hh = hb * 16 + r;                                 // head inside the group
   const bool row_ok = r < ma.rows_per_token && hh < group;
   const int head = kvh * group + min(hh, group - 1);
-  const int pos = uniform(a.positions[token]);
+  // Fused form: the last wave does not walk; it prepares the query rows for the others.
+  // In the first split the wave before it does not walk either: it takes the new key,
+  // side by side with the last wave's work on the queries.  What those two need from
+  // memory is asked for first of all, before anything else is worked out: the head
+  // vector and the norm weight at once, cos and sin as soon as the position is here.
   const bool new_key = FUSED && args.kv_in_row > 0;           // the step's own key is not in the cache yet
+  const bool adds_new = new_key && split == 0;                // this workgroup brings the new key in
+  const bool prep_wave = FUSED && wave == NW - 1;
+  const bool key_wave = adds_new && wave == NW - 2;
+  const bool walker = !prep_wave && !key_wave;
+  const int pos_lane = a.positions[token];
+  bf16x8 kq[KS];            // the head vector such a wave prepares: query rows, or the new key
+  f32x4 cs[KS][4];          // cos (2 x 4) and sin (2 x 4) of the lane's elements
+  f32x4 pw[KS][2];          // norm weight
+  const float* prep_weight = nullptr;
+  if constexpr (FUSED) {
+    if (!walker) {
+      prep_weight = prep_wave ? args.q_weight : args.k_weight;
+      const bf16_t* src = args.qkv + (int64_t)token * ((a.nq + 2 * args.kv_in_row) * HD) +
+                          (int64_t)(prep_wave ? head : a.nq + kvh) * HD + g * (HD / 4);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        kq[s] = *(const bf16x8*)(src + s * 8);
+        if (prep_weight) {
+          pw[s][0] = *(const f32x4*)(prep_weight + g * (HD / 4) + s * 8);
+          pw[s][1] = *(const f32x4*)(prep_weight + g * (HD / 4) + s * 8 + 4);
+        }
+      }
+    }
+  }
+  const int pos = uniform(pos_lane);
+  if constexpr (FUSED) {
+    if (!walker && args.cos != nullptr) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int64_t i = (int64_t)pos * (HD / 2) + (g & 1) * (HD / 4) + s * 8;
+        cs[s][0] = *(const f32x4*)(args.cos + i);
+        cs[s][1] = *(const f32x4*)(args.cos + i + 4);
+        cs[s][2] = *(const f32x4*)(args.sin + i);
+        cs[s][3] = *(const f32x4*)(args.sin + i + 4);
+      }
+    }
+  }
   const int last = new_key ? pos - 1 : pos;                   // last key walked from the cache
   const int lo = (a.window > 0) ? max(0, pos - a.window + 1) : 0;
-  const bool adds_new = new_key && split == 0;                // this workgroup brings the new key in
-
   // chunks of this split: the arithmetic of attention_merge (from pos, not from last)
   const int c_first = lo / kChunk, c_last = pos / kChunk;
   const int per = (c_last - c_first + ma.num_splits) / ma.num_splits;
@@ -129,11 +168,6 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     return;
   }
 
-  // fused form: the last wave does not walk; it prepares the query rows for the others.
-  // In the first split the wave before it does not walk either: it takes the new key,
-  // side by side with the last wave's work on the queries.
-  const bool prep_wave = FUSED && wave == NW - 1;
-  const bool key_wave = adds_new && wave == NW - 2;
   const int walkers = FUSED ? NW - 1 - (adds_new ? 1 : 0) : NW;
 
   TileState<HD> t;
@@ -154,35 +188,12 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     const int row_width = (a.nq + 2 * args.kv_in_row) * HD;
     const bf16_t* row = args.qkv + (int64_t)token * row_width;
     const bool rotate = args.cos != nullptr;
-    const bool walker = !prep_wave && !key_wave;
     if (walker) {
       cur.start(key_begin);
       if (key_begin < key_end) load_kv_block<HD, true>(A, a, table, cur, kvh, key_begin, stride, r, g);
     }
-    // the head vector a wave that does not walk prepares: the query rows, or the new key
-    // (the same in all 16 rows)
-    bf16x8 kq[KS];
     if (!walker) {
-      const float* weight = prep_wave ? args.q_weight : args.k_weight;
-      const bf16_t* src = row + (int64_t)(prep_wave ? head : a.nq + kvh) * HD + g * (HD / 4);
-      f32x4 cs[KS][4];          // cos (2 x 4) and sin (2 x 4) of the lane's elements
-      f32x4 w[KS][2];
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        kq[s] = *(const bf16x8*)(src + s * 8);
-        if (rotate) {
-          const int64_t i = (int64_t)pos * (HD / 2) + (g & 1) * (HD / 4) + s * 8;
-          cs[s][0] = *(const f32x4*)(args.cos + i);
-          cs[s][1] = *(const f32x4*)(args.cos + i + 4);
-          cs[s][2] = *(const f32x4*)(args.sin + i);
-          cs[s][3] = *(const f32x4*)(args.sin + i + 4);
-        }
-        if (weight) {
-          w[s][0] = *(const f32x4*)(weight + g * (HD / 4) + s * 8);
-          w[s][1] = *(const f32x4*)(weight + g * (HD / 4) + s * 8 + 4);
-        }
-      }
-      prepare_head<HD>(kq, prep_wave ? row_ok : true, weight != nullptr, w, args.eps, cs, rotate, g);
+      prepare_head<HD>(kq, prep_wave ? row_ok : true, prep_weight != nullptr, pw, args.eps, cs, rotate, g);
       if (prep_wave) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) s_q[s][lane] = kq[s];
