@@ -195,7 +195,9 @@ def test_norm_linear(ops, gpu_device, dtype, silu, M, N, K):
 @pytest.mark.parametrize("silu", [False, True])
 @pytest.mark.parametrize("M,W,K,N", [(8, 1024, 2048, 4096), (1, 1024, 3072, 6144), (64, 1024, 2048, 4096),
                                      (33, 520, 1096, 1392), (16, 1000, 2056, 112), (17, 4096, 512, 160),
-                                     (7, 2048, 4096, 528), (40, 1000, 520, 2000)])
+                                     (7, 2048, 4096, 528), (40, 1000, 520, 2000),
+                                     (8, 1280, 1024, 512), (4, 1536, 512, 1024), (2, 3000, 520, 264),
+                                     (3, 1024, 2048, 4096), (12, 1024, 3072, 6144)])
 def test_linear_into_stream_then_norm_linear(ops, gpu_device, silu, M, W, K, N):
     """The norm split over two products (bfloat16 only): the first adds bf16(x Wo^T) into
     the stream [M, W] in place and prepares the rows, the second is norm_linear over them.

@@ -47,10 +47,12 @@ int gemm_direct_row_tiles(int M, int N, int most) {
 }
 
 // Columns per workgroup for a plain or tail product of up to 16 rows: fewer than 16 while
-// that gives the chip's 256 compute units more workgroups to share the weight among.
+// that gives the chip's 256 compute units more workgroups to share the weight among, and
+// never more than 256 of them (the slices of the tail form's sums of squares are one per
+// workgroup, and the product that follows holds 256 of them in its lanes).
 int gemm_direct_columns(int M, int N) {
   if (M > 16 || (N + 15) / 16 >= 192) return 16;
-  return (N + 7) / 8 >= 192 ? 8 : 4;
+  return N <= 1024 ? 4 : N <= 2048 ? 8 : 16;
 }
 
 // Fused norm in front (at most 16 rows): the operand is built in registers, nothing packed.
