@@ -159,6 +159,13 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   // issued unconditionally (a missing page reads page 0 and is zeroed when stored to
   // LDS), so nothing but the barrier stands between them and the work on the block.
   constexpr bool kEven = (2 * KS) % 4 == 0, vEven = (2 * DB) % 4 == 0;
+  // Values, wide form (head sizes in steps of 64): a block's values are DB * 16 head
+  // elements times 32 keys, 64 bytes a row of the transposed page: a lane fetches 8 keys
+  // of one row in a 16-byte load (lane % 4 = which 8 keys, lane / 4 and the instruction =
+  // which row) instead of 4 keys in an 8-byte one, half the load instructions, and the two
+  // groups of 4 keys go to their lanes' slots in LDS, every lane of a store to a bank of
+  // its own.
+  constexpr bool kWideV = DB % 4 == 0;
   // kAhead blocks are on their way from memory while one is worked on.  More than one
   // was measured and does not pay: the registers they take cost a resident wave, and it
   // is the number of resident waves (four per SIMD up to head size 128) that hides the
@@ -167,7 +174,9 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   struct Fetched {
     bf16x8 k[KQ];
     bf16x4 v[VQ];
+    bf16x8 vw[kWideV ? DB / 4 : 1];             // wide form: 8 keys of one head element each
     bool kvalid[KQ], vvalid[VQ];                // wave-uniform but for the head size's tail
+    bool vwvalid;                               // wide form: this lane's half of the block
   };
   Fetched ring[kAhead];
   // address = head base + page * page stride (scalar) + position in page (scalar)
@@ -187,6 +196,13 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
     k_blk[i] = q / KS;
     k_dim_ok[i] = KS * 32 == HD || g * 8 * KS + s0 * 8 < HD;
     k_lane[i] = 2u * (r * HD + min(g * 8 * KS + s0 * 8, HD - 8));
+  }
+  const int vw_q = lane % 4;                          // keys vw_q * 8 .. + 7 of the block
+  unsigned vw_lane[kWideV ? DB / 4 : 1];
+  if constexpr (kWideV) {
+#pragma unroll
+    for (int i = 0; i < DB / 4; ++i)
+      vw_lane[i] = 2u * ((((i * 4 + wave) * 16 + lane / 4) * P) + (vw_q % 2) * 8);
   }
 #pragma unroll
   for (int i = 0; i < VQ; ++i) {
@@ -213,10 +229,18 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
       f.kvalid[i] = (k_blk[i] ? page1 : page0) >= 0 && k_dim_ok[i];
       f.k[i] = *(const bf16x8*)((const char*)(k_blk[i] ? kb1 : kb0) + lane_offset(k_lane[i]));
     }
+    if constexpr (kWideV) {
+      const bool second = vw_q >= 2;             // the block's second 16 keys
+      f.vwvalid = (second ? page1 : page0) >= 0;
+      const char* vb = (const char*)(second ? vb1 : vb0);
 #pragma unroll
-    for (int i = 0; i < VQ; ++i) {
-      f.vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
-      f.v[i] = *(const bf16x4*)((const char*)(v_blk[i] ? vb1 : vb0) + lane_offset(v_lane[i]));
+      for (int i = 0; i < DB / 4; ++i) f.vw[i] = *(const bf16x8*)(vb + vw_lane[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VQ; ++i) {
+        f.vvalid[i] = (v_blk[i] ? page1 : page0) >= 0;
+        f.v[i] = *(const bf16x4*)((const char*)(v_blk[i] ? vb1 : vb0) + lane_offset(v_lane[i]));
+      }
     }
     cur.start(kb + 32);
   };
@@ -227,6 +251,19 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
     for (int i = 0; i < KQ; ++i)
       if (kEven || wave + 4 * i < 2 * KS)
         k_lds[buf][wave + 4 * i][lane] = f.kvalid[i] ? f.k[i] : zero8;
+    if constexpr (kWideV) {
+      // keys vw_q*8 .. +3 belong to lane group (vw_q % 2) * 2, the next four to the group
+      // after it, in the half of the slot that the 16-key half of the block has
+#pragma unroll
+      for (int i = 0; i < DB / 4; ++i) {
+        const bf16x8 x = f.vwvalid ? f.vw[i] : zero8;
+        const bf16x4 lo = {x[0], x[1], x[2], x[3]}, hi = {x[4], x[5], x[6], x[7]};
+        bf16x4* slot = (bf16x4*)&v_lds[buf][i * 4 + wave][(vw_q % 2) * 32 + lane / 4];
+        slot[vw_q / 2] = lo;
+        slot[32 + vw_q / 2] = hi;                 // 16 lanes further: the next lane group
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < VQ; ++i)
       if (vEven || wave + 4 * i < 2 * DB)
