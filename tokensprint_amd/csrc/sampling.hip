@@ -2,7 +2,9 @@
 // argmax(logit/T - log E) with E ~ Exp(1), which picks token i with probability
 // softmax(logits/T)[i].  The noise of (row, vocabulary index) comes from a counter hash
 // keyed per row, so a token does not depend on what else is in the batch.
+#include <mutex>
 #include "common.h"
+#include "sampling_static.h"
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
@@ -111,5 +113,59 @@ extern "C" int ts_sample(const float* logits, const float* temperature, const ui
   hipLaunchKernelGGL(pick_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out,
                      slices);
   TS_CHECK_LAUNCH("sample");
+  return 0;
+}
+
+// ---------------------------------------------------------------- no allocation
+// The slice winners of ts_sample_static: value and index of each, in one device array of
+// the library instead of a workspace of the caller's.  In host code `scratch` is only a
+// handle for hipGetSymbolAddress; the address kernels get is looked up once per device.
+constexpr int kStaticWinners = 1 << 16;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)kStaticWinners * 8];
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+extern "C" int ts_sample_static_capacity() { return kStaticWinners; }
+
+// The device address of `scratch` on the current device (each GPU has its own copy).
+static int static_scratch(void** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) TS_FAIL("sample_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices)
+    TS_FAIL("sample_static: device %d beyond the %d this library keeps scratch for", device,
+            kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      TS_FAIL("sample_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  return 0;
+}
+
+extern "C" int ts_sample_static(const float* logits, const float* temperature,
+                                const uint64_t* keys, int* out, int rows, int vocab,
+                                hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (vocab <= 0) TS_FAIL("sample_static: vocab=%d", vocab);
+  const int slices = (vocab + kSlice - 1) / kSlice;
+  if ((int64_t)rows * slices > kStaticWinners)
+    TS_FAIL("sample_static: %d rows x %d slices of the vocabulary exceed the %d slice "
+            "winners the library's scratch holds; use ts_sample with a workspace",
+            rows, slices, kStaticWinners);
+  void* base = nullptr;
+  if (static_scratch(&base) != 0) return -1;
+  float* part_v = (float*)base;
+  int* part_i = (int*)((unsigned char*)base + (size_t)kStaticWinners * 4);
+  hipLaunchKernelGGL(pick_slices_kernel<true>, dim3(rows, slices), dim3(256), 0, stream, logits,
+                     temperature, keys, part_v, part_i, vocab);
+  hipLaunchKernelGGL(pick_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out,
+                     slices);
+  TS_CHECK_LAUNCH("sample_static");
   return 0;
 }
