@@ -1,28 +1,21 @@
-"""Prints the registered models grouped by family (the reference's
-model_registry.py:8-22) and the registered architectures."""
+"""Lists the models this engine knows by name, family by family, and the architectures
+it can build (output in the manner of the reference's model_registry.py:8-22)."""
 
 from __future__ import annotations
 
-from collections import defaultdict
-
-from tokensprint_amd.config import (all_registered_models, architecture_names,
-                                    get_model_family, get_model_repo_id)
+from tokensprint_amd.config import architecture_names, models_by_family
 
 
-def main() -> None:
-    families: dict[str, list[str]] = defaultdict(list)
-    for model in all_registered_models(newest_first=False):
-        families[get_model_family(model)].append(model)
+def listing() -> str:
+    families = models_by_family()
     if not families:
-        print("No models are currently registered.")
-        return
-    print("Registered models:")
-    for family in sorted(families):
-        print(f"\n{family}:")
-        for model in families[family]:
-            print(f"  - {model} ({get_model_repo_id(model)})")
-    print("\nArchitectures: " + ", ".join(architecture_names()))
+        return "No models are currently registered."
+    lines = ["Registered models:"]
+    for family, models in sorted(families.items()):
+        lines += ["", f"{family}:"] + [f"  - {m.short} ({m.repo_id})" for m in models]
+    lines += ["", "Architectures: " + ", ".join(architecture_names())]
+    return "\n".join(lines)
 
 
 if __name__ == "__main__":
-    main()
+    print(listing())

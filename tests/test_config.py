@@ -91,7 +91,9 @@ def test_named_models_resolve_short_and_long():
     assert model_is_registered("qwen3-8b") and model_is_registered("qwen/qwen3-32b")
     assert not model_is_registered("meta-llama/qwen3-0.6b")
     assert get_model_family("qwen3-8b") == "qwen"
-    assert set(get_models_from_family("qwen")) == set(all_registered_models())
+    assert set(get_models_from_family("qwen")) | set(get_models_from_family("tiny")) \
+        == set(all_registered_models())
+    assert get_models_from_family("qwen", newest_first=False)[0] == "qwen3-0.6b"
     with pytest.raises(ValueError, match=r"Unsupported model_name 'nope'. Available models: \[.*qwen/qwen3-0.6b"):
         resolve_model_name("nope")
 
@@ -103,3 +105,10 @@ def test_named_0_6b_matches_the_reference_factory():
             c.vocab_size, c.num_layers, c.max_position, c.rope_theta, c.rms_norm_eps,
             c.tie_word_embeddings) == (1024, 16, 8, 128, 3072, 151_936, 28, 40960,
                                        1_000_000.0, 1e-6, True)
+
+
+def test_tiny_presets_are_the_tiny_test_configurations():
+    from helpers import TINY_A, TINY_B
+    assert resolve_model_name("tiny/tiny-b") == "tiny-b" and not model_is_registered("qwen/tiny-a")
+    for name, cfg in (("tiny-a", TINY_A), ("tiny-b", TINY_B)):
+        assert Qwen3Config.from_dict(load_named_config(name)) == Qwen3Config.from_dict(cfg)

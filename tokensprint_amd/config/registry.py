@@ -9,7 +9,6 @@ under config/presets, so no size stands in code.
 from __future__ import annotations
 
 import json
-from collections import defaultdict
 from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Callable
@@ -25,9 +24,23 @@ class Architecture:
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
-_MODEL_PRESETS: dict[str, Path] = {}
-_MODEL_FAMILY: dict[str, str] = {}
-_FAMILY_MODELS: dict[str, list[str]] = defaultdict(list)
+
+
+@dataclass(frozen=True)
+class NamedModel:
+    """A model known by name: `short` alone or `family/short` (its repository id)."""
+
+    family: str
+    short: str
+    preset: Path                             # a config.json kept as data
+
+    @property
+    def repo_id(self) -> str:
+        return f"{self.family}/{self.short}"
+
+
+_NAMED: dict[str, NamedModel] = {}           # short name -> model, in order of registration
+_presets_read = False
 
 
 def register_architecture(name: str, *, parse_config, build_spec) -> None:
@@ -54,71 +67,82 @@ def architecture_names() -> list[str]:
     return sorted(_ARCHITECTURES)
 
 
+# ------------------------------------------------------------------ named models
+# Behaviour of engine/models/_registry.py:130-151,194-263: a short name is unique over
+# all families, `family/short` names the same model, an unknown name is an error that
+# lists what there is.  Kept here as one table and one lookup.
+
+
 def register_named_model(family: str, name: str, preset: Path) -> None:
-    """engine/models/_registry.py:130-151: duplicates are rejected."""
-    if name in _MODEL_PRESETS:
+    if name in _NAMED:
         raise ValueError(f"Model {name} already registered.")
-    _MODEL_PRESETS[name] = Path(preset)
-    _MODEL_FAMILY[name] = family
-    _FAMILY_MODELS[family].append(name)
+    _NAMED[name] = NamedModel(family, name, Path(preset))
 
 
-def _register_presets() -> None:
-    if _MODEL_PRESETS:
-        return
-    index = json.loads((_PRESET_DIR / "index.json").read_text())
-    for family, names in index.items():
-        for name in names:
-            register_named_model(family, name, _PRESET_DIR / f"{name}.json")
+def _named() -> dict[str, NamedModel]:
+    global _presets_read
+    if not _presets_read:
+        _presets_read = True
+        for family, names in json.loads((_PRESET_DIR / "index.json").read_text()).items():
+            for name in names:
+                if name not in _NAMED:
+                    register_named_model(family, name, _PRESET_DIR / f"{name}.json")
+    return _NAMED
+
+
+def lookup(model_name: str) -> NamedModel:
+    """The model `model_name` means, given as `short` or as `family/short`."""
+    table = _named()
+    family, _, short = model_name.rpartition("/")
+    found = table.get(short)
+    if found is None or (family and family != found.family):
+        known = ", ".join(sorted(m.repo_id for m in table.values()))
+        raise ValueError(f"Unsupported model_name '{model_name}'. Available models: [{known}]")
+    return found
 
 
 def resolve_model_name(model_name: str) -> str:
-    """Short name, or `family/short` when the short name belongs to that family."""
-    _register_presets()
-    if model_name in _MODEL_PRESETS:
-        return model_name
-    if "/" in model_name:
-        family, short = model_name.split("/", 1)
-        if short in _MODEL_PRESETS and _MODEL_FAMILY.get(short) == family:
-            return short
-    available = ", ".join(sorted(all_registered_repo_ids()))
-    raise ValueError(f"Unsupported model_name '{model_name}'. Available models: [{available}]")
+    return lookup(model_name).short
 
 
 def model_is_registered(model_name: str) -> bool:
     try:
-        resolve_model_name(model_name)
-        return True
+        lookup(model_name)
     except ValueError:
         return False
+    return True
 
 
 def get_model_family(model: str) -> str:
-    return _MODEL_FAMILY[resolve_model_name(model)]
+    return lookup(model).family
 
 
 def get_model_repo_id(model: str) -> str:
-    name = resolve_model_name(model)
-    return f"{_MODEL_FAMILY[name]}/{name}"
+    return lookup(model).repo_id
+
+
+def models_by_family() -> dict[str, list[NamedModel]]:
+    """Every named model under its family, families and models in order of registration."""
+    out: dict[str, list[NamedModel]] = {}
+    for m in _named().values():
+        out.setdefault(m.family, []).append(m)
+    return out
 
 
 def get_models_from_family(family: str, newest_first: bool = True) -> list[str]:
-    _register_presets()
-    models = list(_FAMILY_MODELS[family])
-    return models[::-1] if newest_first else models
+    names = [m.short for m in models_by_family().get(family, [])]
+    return names[::-1] if newest_first else names
 
 
 def all_registered_models(newest_first: bool = True) -> list[str]:
-    _register_presets()
-    models = list(_MODEL_PRESETS)
-    return models[::-1] if newest_first else models
+    names = list(_named())
+    return names[::-1] if newest_first else names
 
 
 def all_registered_repo_ids(newest_first: bool = True) -> list[str]:
-    return [f"{_MODEL_FAMILY[n]}/{n}" for n in all_registered_models(newest_first)]
+    return [_NAMED[n].repo_id for n in all_registered_models(newest_first)]
 
 
 def load_named_config(model_name: str) -> dict:
     """The raw config.json dict of a named model."""
-    name = resolve_model_name(model_name)
-    return json.loads(_MODEL_PRESETS[name].read_text())
+    return json.loads(lookup(model_name).preset.read_text())
