@@ -37,24 +37,6 @@ def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, m
     return model, LLMEngine(model, config)
 
 
-def weight_bytes(model) -> int:
-    """Bytes of every weight a decode step reads once (a tied head is counted once;
-    of the embedding table only the head's use is counted when tied)."""
-    seen, total = set(), 0
-    for block in model.blocks:
-        for t in (block.mixer.w_qkv, block.mixer.w_o, block.mixer.w_qnorm, block.mixer.w_knorm,
-                  block.feed_forward.w_gate_up, block.feed_forward.w_down,
-                  block.mixer_norm.weight, block.ffn_norm.weight):
-            if t is not None and t.data_ptr() not in seen:
-                seen.add(t.data_ptr())
-                total += t.numel() * t.element_size()
-    for t in (model.head.weight, model.final_norm.weight):
-        if t.data_ptr() not in seen:
-            seen.add(t.data_ptr())
-            total += t.numel() * t.element_size()
-    return total
-
-
 def decode_run(engine, batch, prompt_len, steps, warmup, vocab):
     """Prefill `batch` prompts, then time exactly `steps` decode steps."""
     import torch
@@ -144,7 +126,7 @@ def main() -> int:
                           "tok_per_s": round(2048 / sec, 1)}))
         return 0
     model, engine = make_engine(raw, args.dtype, layers, args.batch, ctx_len, 2048, page)
-    wbytes = weight_bytes(model)
+    wbytes = model.step_weight_bytes()   # every weight a decode step reads, each once
     kv_per_token = 2 * layers * raw["num_key_value_heads"] * raw["head_dim"] * item
 
     dt, mean_tokens = decode_run(engine, args.batch, args.prompt_len, args.steps, args.warmup,

@@ -31,6 +31,9 @@ def parse_args(argv=None):
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--max-input-len", type=int, default=1024)
     ap.add_argument("--max-output-len", type=int, default=1024)
+    ap.add_argument("--min-input-len", type=int, default=100,
+                    help="prompt lengths are uniform in [min, max]; equal values fix them")
+    ap.add_argument("--min-output-len", type=int, default=100)
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--enforce-eager", type=_bool, default=False)
     ap.add_argument("--chunked-prefill", type=_bool, default=True)
@@ -46,11 +49,16 @@ def parse_args(argv=None):
 
 
 def make_workload(args):
-    """benchmark.py:54-63 of the reference."""
-    prompts = [[randint(0, args.max_prompt_token_id) for _ in range(randint(100, args.max_input_len))]
-               for _ in range(args.num_seqs)]
-    output_lens = [randint(100, args.max_output_len) for _ in range(args.num_seqs)]
-    return prompts, output_lens
+    """The reference's synthetic workload (benchmark.py:54-63): per request a prompt of
+    uniformly random token ids and length, and a uniformly random number of tokens to
+    generate; the lower bounds, fixed at 100 there, are options here."""
+    lo_in, lo_out = min(args.min_input_len, args.max_input_len), \
+        min(args.min_output_len, args.max_output_len)
+    prompts = []
+    for _ in range(args.num_seqs):
+        length = randint(lo_in, args.max_input_len)
+        prompts.append([randint(0, args.max_prompt_token_id) for _ in range(length)])
+    return prompts, [randint(lo_out, args.max_output_len) for _ in range(args.num_seqs)]
 
 
 def main(args) -> None:
@@ -63,18 +71,19 @@ def main(args) -> None:
     seed(0)
     prompts, output_lens = make_workload(args)
     if args.model_dir is not None:
-        model_cfg, model = load_model(args.model_dir, args.dtype, "cuda:0")
+        _, model = load_model(args.model_dir, args.dtype, "cuda:0")
         model_dir = str(args.model_dir)
     else:
         raw = load_named_config(args.model_name)
         if args.layers:
             raw["num_hidden_layers"] = args.layers
-        model_cfg, model = random_model(raw, 0, args.dtype, "cuda:0")
+        _, model = random_model(raw, 0, args.dtype, "cuda:0")
         model_dir = tempfile.gettempdir()
-    max_model_len = args.max_model_len or int(model_cfg.max_position)
-    if max_model_len > model_cfg.max_position:
-        raise ValueError(f"max_model_len cannot exceed the model's {model_cfg.max_position}")
-    limit = min(args.max_prompt_token_id, model_cfg.vocab_size - 1)
+    spec = model.spec
+    max_model_len = args.max_model_len or int(spec.max_position)
+    if max_model_len > spec.max_position:
+        raise ValueError(f"max_model_len cannot exceed the model's {spec.max_position}")
+    limit = min(args.max_prompt_token_id, spec.vocab_size - 1)
     prompts = [[min(t, limit) for t in p] for p in prompts]
     llm = LLMEngine(model, Config(
         model=model_dir, enforce_eager=args.enforce_eager, max_model_len=max_model_len,
@@ -89,8 +98,10 @@ def main(args) -> None:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     total = sum(output_lens)
+    prompt_tokens = sum(len(p) for p in prompts)
     print(f"[tokensprint_amd] Total: {total}tok, Time: {elapsed:.2f}s, "
-          f"Throughput: {total / elapsed:.2f}tok/s, preemptions: {llm.scheduler.num_preemptions}")
+          f"Throughput: {total / elapsed:.2f}tok/s, prompt tokens: {prompt_tokens}, "
+          f"pages: {llm.config.num_kvcache_blocks}, preemptions: {llm.scheduler.num_preemptions}")
 
 
 if __name__ == "__main__":

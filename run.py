@@ -18,6 +18,7 @@ from pathlib import Path
 
 logging.basicConfig(level=logging.INFO,
                     format="%(asctime)s %(levelname)s %(name)s: %(message)s", force=True)
+log = logging.getLogger("run")
 
 
 def _bool(text: str) -> bool:
@@ -76,20 +77,27 @@ def main(args) -> None:
                            dtype)
     elif model_dir is None:
         model_dir = args.cache_dir / get_model_repo_id(args.model_name).split("/")[-1]
-    model_cfg, model = load_model(model_dir, dtype, "cuda:0")
+    _, model = load_model(model_dir, dtype, "cuda:0")
+    spec = model.spec           # sizes and the end-of-sequence token come from the model as
+                                # built, whatever architecture config.json named
 
     tokenizer = None
     if args.prompt_ids is None:
-        from transformers import AutoTokenizer
-        tokenizer = AutoTokenizer.from_pretrained(str(model_dir))
+        from tokensprint_amd.tokenizer import describe, load_tokenizer
+        tokenizer = load_tokenizer(model_dir)
+        log.info("tokenizer: %s", describe(tokenizer))
         prompt = args.prompt
     else:
         prompt = [int(t) for t in args.prompt_ids.split(",")]
-    eos = tokenizer.eos_token_id if tokenizer is not None else (
-        model_cfg.eos_token_id if model_cfg.eos_token_id is not None else -1)
+    # end of sequence: the tokenizer's, as the reference's run.py:53; without a tokenizer
+    # the one config.json names (ModelSpec.eos_token_id), else none
+    if tokenizer is not None:
+        eos = tokenizer.eos_token_id
+    else:
+        eos = spec.eos_token_id if spec.eos_token_id is not None else -1
 
     config = Config(
-        model=str(model_dir), max_model_len=args.max_model_len or int(model_cfg.max_position),
+        model=str(model_dir), max_model_len=args.max_model_len or int(spec.max_position),
         eos=eos, dtype=dtype, enforce_eager=args.enforce_eager,
         kvcache_block_size=args.page_size, num_kvcache_blocks=args.num_pages,
         max_num_batched_tokens=args.max_num_batched_tokens, max_num_seqs=args.max_num_seqs,

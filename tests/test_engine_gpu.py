@@ -143,3 +143,38 @@ def test_captured_decode_steps_with_many_requests(setup):
         if step % 2 == 0:                     # eager work between replays
             rc = live[0][0]
             runner.step([StepEntry(rc, toks[:3], 0, [2])])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_eps_of_the_per_head_norms_shows(name, dtype, tmp_path, gpu_device):
+    """Random weights give head vectors far above eps, so a wrong eps in the q/k norm
+    would pass every other test.  Here the q and k projections are scaled down until a
+    head vector's mean square is near eps; the logits then depend on eps (the plain
+    implementation with another eps is far outside the tolerance) and the engine must
+    agree with the plain implementation at the configured one."""
+    import json
+    from safetensors.torch import save_file
+    from tokensprint_amd.weights import random_tensors
+    cfg, seed, page = TINY[name]
+    cfg = dict(cfg, torch_dtype="float32" if dtype == torch.float32 else "bfloat16")
+    tensors = random_tensors(cfg, seed, dtype=torch.float32)
+    for key in tensors:
+        if key.endswith(("q_proj.weight", "k_proj.weight")):
+            tensors[key] = tensors[key] * 0.01
+    tensors = {k: v.to(dtype).contiguous() for k, v in tensors.items()}
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    pcfg, w = plain.read_model_dir(tmp_path)
+    _, model = load_model(tmp_path, dtype, gpu_device)
+    requests = {"a": random_prompt(50, cfg["vocab_size"], 1), "b": random_prompt(37, cfg["vocab_size"], 2)}
+    ref = {rid: plain.forward_logits(pcfg, w, t) for rid, t in requests.items()}
+    rtol, atol = TOL[dtype]
+    other = plain.forward_logits({**pcfg, "rms_norm_eps": pcfg["rms_norm_eps"] * 10}, w, requests["a"])
+    # only the per-head norms can make this difference large: the block norms see the
+    # same change in every other test's weights and move the logits far less.  In
+    # float32 a wrong eps is 20 tolerances away; bfloat16's tolerance hides most of it
+    margin = 20 if dtype == torch.float32 else 1.5
+    assert (other - ref["a"]).abs().max() > margin * (atol + rtol * ref["a"].abs().max())
+    col = drives.drive_prefill_then_decode(runner_for(model, page, 128 // page), requests, tail=12)
+    drives.compare(col, ref, rtol, atol)

@@ -138,10 +138,44 @@ def test_temperature_sampling_does_not_depend_on_the_batch(setup):
     assert third != together
 
 
-def test_bfloat16_generation_agrees_mostly(setup, tmp_path, gpu_device):
+def test_pool_sized_from_free_memory_and_warm_engine(setup):
+    """num_kvcache_blocks left at -1: the pool is sized from what a measured largest step
+    and the captured graphs leave; every decode bucket is captured before a request."""
+    cfg, d, model, page, prompts, expected = setup
+    engine = engine_for(model, d, torch.float32, kvcache_block_size=page, num_kvcache_blocks=-1,
+                        max_model_len=cfg["max_position_embeddings"], max_num_seqs=24)
+    pages = engine.config.num_kvcache_blocks
+    assert pages == 24 * (-(-cfg["max_position_embeddings"] // page) + 1)   # capped: tiny model
+    assert set(engine.runner.graphs) == {1, 2, 4, 8, 16, 24}
+    assert engine.generate(prompts, GREEDY, use_tqdm=False) == expected
+    assert all(p.num_used == 0 for p in engine.runner.manager.pools)
+
+
+def test_bfloat16_logits_of_the_generated_tokens(setup, gpu_device):
+    """bfloat16 through the entry point's own steps (prefill in portions, captured decode):
+    the fp32 plain tokens are forced, and the logits every step returns are compared with
+    the plain logits at that position."""
+    from tokensprint_amd.engine import StepEntry
     cfg, d, _, page, prompts, expected = setup
+    pcfg, w = plain.read_model_dir(d)
     _, model = load_model(d, torch.bfloat16, gpu_device)
-    engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=cfg["max_position_embeddings"])
-    got = engine.generate(prompts, GREEDY, use_tqdm=False)
-    first = sum(g[0] == e[0] for g, e in zip(got, expected))
-    assert first >= len(prompts) - 1          # the first token hangs on no earlier choice
+    engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page,
+                        max_model_len=cfg["max_position_embeddings"])
+    runner = engine.runner
+    for prompt, completion in zip(prompts, expected):
+        tokens = prompt + completion
+        ref = plain.forward_logits(pcfg, w, tokens)
+        rc = runner.manager.admit("r")
+        got = {}
+        pos = 0
+        for n in [min(7, len(prompt))] * (len(prompt) // 7) + [len(prompt) % 7] + [1] * len(completion):
+            if n == 0:
+                continue
+            runner.manager.extend(rc, pos + n)
+            entry = StepEntry(rc, tokens[pos:pos + n], pos, [n - 1])
+            got[pos + n - 1] = runner.step([entry])[0].float().cpu()
+            pos += n
+        runner.manager.free(rc)
+        for p, row in got.items():
+            torch.testing.assert_close(row, ref[p], rtol=3e-2, atol=3e-2)
+    assert runner.graphs                 # the single-token steps were replays

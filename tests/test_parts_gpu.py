@@ -124,7 +124,11 @@ def test_attention_and_swiglu_and_block_parts(gpu_device, dtype, window):
 class ToyDecayMixer(Mixer):
     """State s (one vector per request): s <- decay * s + x_t; output W s.  Tokens of a
     request must be taken in order, and the state lives in the request's slot between
-    steps.  Written with torch operations: it stands for a part someone brings along."""
+    steps.  Written with torch operations: it stands for a part someone brings along.
+    It reads the slot ids back to the host, so it cannot run inside a captured graph and
+    says so."""
+
+    capturable = False
 
     def __init__(self, params, ctx):
         super().__init__(params, ctx)
@@ -152,6 +156,24 @@ class ToyDecayMixer(Mixer):
                 out[t] = (self.w.float() @ s).to(h.dtype)
             first += n
         return out
+
+
+class ToyDecayMixerOnDevice(ToyDecayMixer):
+    """The same mixer with a decode step (one token per entry) that touches device tensors
+    only, so it may be captured: the state rows of the step's slots are gathered, updated
+    and scattered back.  Idle lanes of a captured batch carry the slot no request owns."""
+
+    capturable = True
+
+    def forward(self, h, batch, cache, write_cache):
+        if batch.max_q_len > 1:
+            return super().forward(h, batch, cache, write_cache)
+        slots = batch.slot_ids.long()
+        s = cache.state.index_select(0, slots)
+        s = torch.where((batch.positions == 0)[:, None], torch.zeros_like(s), s)
+        s = s * self.decay + h.float()
+        cache.state.index_copy_(0, slots, s)
+        return (s @ self.w.float().T).to(h.dtype)
 
 
 class ToyTop1FeedForward(FeedForward):
@@ -199,7 +221,8 @@ def toy_spec(raw):
     layers = (
         LayerSpec("pre_norm", attn("l0.attn.", "offset"), PartSpec("swiglu", {"prefix": "l0.ffn.", "inner_dim": 40}),
                   norm("l0.n1"), norm("l0.n2")),
-        LayerSpec("pre_norm", PartSpec("toy_decay", {"weight": "l1.mix", "decay": 0.5}),
+        LayerSpec("pre_norm", PartSpec(raw.get("decay_mixer", "toy_decay"),
+                                       {"weight": "l1.mix", "decay": 0.5}),
                   PartSpec("toy_top1", {"prefix": "l1.ffn."}), norm("l1.n1"), norm("l1.n2")),
         LayerSpec("pre_norm", attn("l2.attn.", "rope", own=False), PartSpec("swiglu", {"prefix": "l2.ffn.", "inner_dim": 24}),
                   norm("l2.n1"), norm("l2.n2")),
@@ -218,7 +241,9 @@ def toy_spec(raw):
 
 @pytest.fixture(scope="module")
 def toy_registered():
-    for reg, kind, cls in ((MIXERS, "toy_decay", ToyDecayMixer), (FEED_FORWARDS, "toy_top1", ToyTop1FeedForward),
+    for reg, kind, cls in ((MIXERS, "toy_decay", ToyDecayMixer),
+                           (MIXERS, "toy_decay_on_device", ToyDecayMixerOnDevice),
+                           (FEED_FORWARDS, "toy_top1", ToyTop1FeedForward),
                            (POSITIONS, "toy_offset", ToyOffsetEncoding)):
         register(reg, kind, replace=True)(cls)
     if "ToyForTests" not in _ARCHITECTURES:
@@ -286,7 +311,7 @@ def test_toy_parts_build_and_step(toy_registered, gpu_device):
     assert [type(n).__name__ for n in needs] == ["PagedKVNeed", "SlotStateNeed", "PagedKVNeed", "NoneType"]
     runner = ModelRunner(model, page_size=4, num_pages=40, num_slots=3)
     assert len(runner.storage.groups) == 1 and runner.storage.groups[0].runs == (0, 2)
-    assert runner.storage.views[1].state.shape == (3, 64)
+    assert runner.storage.views[1].state.shape == (3 + 1, 64)     # one row for idle lanes
     g = torch.Generator().manual_seed(0)
     reqs = {rid: torch.randint(0, 97, (n,), generator=g).tolist() for rid, n in (("a", 30), ("b", 19), ("c", 44))}
     ref = {rid: toy_plain(model, toks) for rid, toks in reqs.items()}
@@ -317,3 +342,42 @@ def test_toy_parts_build_and_step(toy_registered, gpu_device):
     for rid in reqs:
         out = torch.stack([got[rid][p] for p in range(len(reqs[rid]))])
         torch.testing.assert_close(out, ref[rid], rtol=2e-4, atol=2e-4)
+
+
+def toy_greedy(model, prompt, n):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(toy_plain(model, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+@pytest.mark.parametrize("mixer", ["toy_decay", "toy_decay_on_device"])
+def test_toy_architecture_generates_through_the_engine(toy_registered, gpu_device, tmp_path, mixer):
+    """The toy architecture behind LLMEngine.generate: scheduler, portions, a pool so small
+    that requests are preempted and recomputed, and captured decode steps.  The mixer
+    that reads its slots back to the host keeps every step eager by declaring itself not
+    capturable; its device-only twin is captured, idle lanes included."""
+    from tokensprint_amd.config import Config, SamplingParams
+    from tokensprint_amd.engine.llm_engine import LLMEngine
+    raw = dict(toy_registered, decay_mixer=mixer)
+    _, model = random_model(raw, seed=5, dtype=torch.float32, device=gpu_device, std=0.2)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 97, (n,), generator=g).tolist() for n in (9, 1, 30, 17, 22)]
+    want = [toy_greedy(model, p, 10) for p in prompts]
+    sp = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+    for pages in (64, 14):
+        engine = LLMEngine(model, Config(
+            model=str(tmp_path), max_model_len=128, dtype=torch.float32, kvcache_block_size=4,
+            num_kvcache_blocks=pages, max_num_seqs=3, max_num_batched_tokens=16,
+            chunked_prefill=True))
+        captured = mixer == "toy_decay_on_device"
+        assert bool(engine.runner.buckets) == captured
+        assert set(engine.runner.graphs) == ({1, 2, 3} if captured else set())
+        assert engine.generate(prompts, sp, use_tqdm=False) == want, pages
+        if pages == 14:
+            assert engine.scheduler.num_preemptions > 0
+        engine.runner.manager.check()
+    with pytest.raises(ValueError, match="fixed-size state"):
+        LLMEngine(model, Config(model=str(tmp_path), max_model_len=128, dtype=torch.float32,
+                                kvcache_block_size=4, num_kvcache_blocks=32, max_num_seqs=3,
+                                enable_prefix_caching=True))

@@ -40,10 +40,15 @@ def test_rms_norm_invariants():
 
 # ------------------------------------------------------------------ rotation
 def test_rope_frequencies():
-    # engine/nn/rope.py:28-29; the reference's tests/test_rope_scaling.py:63-79
-    f = plain.rope_inv_freq(8, 10000.0)
-    assert f[0] == 1.0
-    torch.testing.assert_close(f, torch.tensor([10000.0 ** (-2 * i / 8) for i in range(4)]))
+    # engine/nn/rope.py:28-29; the reference's tests/test_rope_scaling.py:63-79 pins the same
+    # base frequencies.  By hand for head size 8 and base 10^4: 10^(-i), i = 0..3
+    torch.testing.assert_close(plain.rope_inv_freq(8, 10000.0),
+                               torch.tensor([1.0, 0.1, 0.01, 0.001]))
+    f = plain.rope_inv_freq(128, 1e6)
+    assert f.shape == (64,) and f[0] == 1.0 and f.dtype == torch.float32
+    # a geometric sequence that ends one step short of 1/base
+    torch.testing.assert_close(f[1:] / f[:-1], torch.full((63,), 1e6 ** (-1 / 64)))
+    torch.testing.assert_close(f[-1] * 1e6 ** (-1 / 64), torch.tensor(1e-6))
 
 
 def test_rope_position_zero_is_identity_and_norms_are_kept():
@@ -138,20 +143,74 @@ def test_block_is_identity_when_output_projections_are_zero():
     torch.testing.assert_close(hidden, ref)
 
 
+def _mixer_by_hand(h, w, p, pos, *, norm_first, eps, theta=1e4, nq=4, nkv=2, hd=16):
+    """The attention mixer put together here from the pinned pieces, with the per-head norm
+    before the rotation (`norm_first`) or after it."""
+    T = h.shape[0]
+    q = (h @ w[p + "q_proj.weight"].T).view(T, nq, hd)
+    k = (h @ w[p + "k_proj.weight"].T).view(T, nkv, hd)
+    v = (h @ w[p + "v_proj.weight"].T).view(T, nkv, hd)
+    cos, sin = plain.rope_cos_sin(pos, hd, theta)
+    norm = lambda t, name: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w[p + name]
+    if norm_first:
+        q, k = norm(q, "q_norm.weight"), norm(k, "k_norm.weight")
+    q, k = plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin)
+    if not norm_first:
+        q, k = norm(q, "q_norm.weight"), norm(k, "k_norm.weight")
+    o = plain.causal_attention(q, k, v)
+    return o.reshape(T, nq * hd) @ w[p + "o_proj.weight"].T
+
+
 def test_qk_norm_comes_before_the_rotation_and_v_is_untouched():
-    # with unit norm weights every q/k head vector entering the rotation has RMS 1, so
-    # scaling the q projection by 10 cannot change the output; scaling v must scale it
+    # engine/nn/attention.py:178-184.  The rotation keeps a head vector's length, so only
+    # the norm's weight tells the two orders apart: it must differ between the two
+    # elements of a rotated pair.  Both orders are computed here; the plain mixer must be
+    # the first and must not be the second.
     w = weights(TINY_A, 0)
-    ids = random_prompt(8, 256, 1)
-    pos = torch.arange(8)
-    h = rnd(8, 64)
-    kw = dict(num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-9, theta=1e4)
     p = "model.layers.0.self_attn."
-    base = plain.attention_mixer(h, w, p, pos, **kw)
-    w2 = dict(w); w2[p + "q_proj.weight"] = 10 * w[p + "q_proj.weight"]
-    torch.testing.assert_close(plain.attention_mixer(h, w2, p, pos, **kw), base, rtol=1e-4, atol=1e-6)
+    w[p + "q_norm.weight"] = torch.linspace(0.3, 2.5, 16)
+    w[p + "k_norm.weight"] = torch.linspace(1.9, 0.4, 16)
+    pos = torch.arange(8) * 5 + 3
+    h = 4 * rnd(8, 64)
+    kw = dict(num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-6, theta=1e4)
+    got = plain.attention_mixer(h, w, p, pos, **kw)
+    before = _mixer_by_hand(h, w, p, pos, norm_first=True, eps=1e-6)
+    after = _mixer_by_hand(h, w, p, pos, norm_first=False, eps=1e-6)
+    torch.testing.assert_close(got, before, rtol=1e-5, atol=1e-6)
+    assert (got - after).abs().max() > 100 * (got - before).abs().max() + 1e-3
+    # v is neither normed nor rotated: scaling its projection scales the output
     w3 = dict(w); w3[p + "v_proj.weight"] = 10 * w[p + "v_proj.weight"]
-    torch.testing.assert_close(plain.attention_mixer(h, w3, p, pos, **kw), 10 * base, rtol=1e-4, atol=1e-6)
+    torch.testing.assert_close(plain.attention_mixer(h, w3, p, pos, **kw), 10 * got,
+                               rtol=1e-4, atol=1e-6)
+
+
+def test_qk_norm_uses_the_given_eps():
+    # the per-head norms take the same eps as the block norms (config.json has one
+    # rms_norm_eps; the reference's separate qk_norm_eps has the same value,
+    # engine/models/qwen/_archs.py:103,122).  With head vectors whose mean square is near
+    # eps, the value of eps shows in the output.
+    w = weights(TINY_A, 0)
+    p = "model.layers.0.self_attn."
+    pos = torch.arange(8)
+    h = 0.02 * rnd(8, 64)                      # q, k elements of about 3e-3: mean square 1e-5
+    kw = dict(num_heads=4, num_kv_heads=2, head_dim=16, theta=1e4)
+    got = plain.attention_mixer(h, w, p, pos, eps=1e-5, **kw)
+    torch.testing.assert_close(got, _mixer_by_hand(h, w, p, pos, norm_first=True, eps=1e-5),
+                               rtol=1e-5, atol=1e-9)
+    other = _mixer_by_hand(h, w, p, pos, norm_first=True, eps=1e-6)
+    assert (got - other).abs().max() > 1e-2 * got.abs().max()
+    # and the model passes config.json's rms_norm_eps down to them
+    ids = random_prompt(9, 256, 1)
+    small = dict(w)
+    for i in range(2):
+        for name in ("q_proj", "k_proj"):
+            key = f"model.layers.{i}.self_attn.{name}.weight"
+            small[key] = 0.01 * w[key]
+    a = plain.forward_logits({**TINY_A, "rms_norm_eps": 1e-6}, small, ids)
+    b = plain.forward_logits({**TINY_A, "rms_norm_eps": 1e-5}, small, ids)
+    c = plain.forward_logits({**TINY_A, "rms_norm_eps": 1e-5}, w, ids)
+    d = plain.forward_logits({**TINY_A, "rms_norm_eps": 1e-6}, w, ids)
+    assert (a - b).abs().max() > 10 * (c - d).abs().max()
 
 
 def test_logits_depend_on_distances_only():

@@ -156,11 +156,13 @@ class RequestCache:
 
 class CacheManager:
     def __init__(self, groups: list[GroupLayout], page_size: int, num_pages,
-                 num_slots: int) -> None:
-        """`num_pages`: one int for every group, or a list with one int per group."""
+                 num_slots: int, state_runs: tuple[int, ...] = ()) -> None:
+        """`num_pages`: one int for every group, or a list with one int per group.
+        `state_runs`: the runs that keep fixed-size state in the request's slot."""
         if page_size < 1:
             raise ValueError(f"page size must be >= 1, got {page_size}")
         self.groups = list(groups)
+        self.state_runs = tuple(state_runs)
         self.page_size = page_size
         counts = [num_pages] * len(groups) if isinstance(num_pages, int) else list(num_pages)
         if len(counts) != len(groups):
@@ -177,10 +179,17 @@ class CacheManager:
     # keep their hash while free, reference counts for sharing, and never takes the last
     # block of a request from the cache (engine/generation/block_manager.py:72-93,161-211,
     # 406-475).  The same here, over all groups at once; only for models whose groups all
-    # keep every key (a window group gives pages back, so its prefix is not there to share).
+    # keep every key (a window group gives pages back, so its prefix is not there to share)
+    # and that keep nothing else per request: state in a slot is what the whole prefix
+    # made of it, and no page holds a copy to start from.
     def enable_prefix_cache(self) -> None:
         if any(g.window is not None for g in self.groups):
             raise ValueError("prefix caching needs every cache group to keep all keys")
+        if self.state_runs:
+            raise ValueError(
+                f"prefix caching cannot serve runs {list(self.state_runs)}, which keep "
+                "fixed-size state per request: a request that starts behind cached pages "
+                "would start with empty state")
         if self.prefix_index is None:
             self.prefix_index = {}
             for g, pool in enumerate(self.pools):

@@ -7,8 +7,9 @@ page, [runs, num_pages, nkv, hd, P].  One key/value head's part of a page is con
 in both; keys are contiguous along the head size (the reduction of q.k) and values along
 the positions (the reduction of p.v), which is what the matrix-core kernels read without
 a transpose.  A run's view is `LayerCache`.
-Per-request state of fixed size lives in [num_slots, *shape] tensors, one per run
-that asks for it.
+Per-request state of fixed size lives in [num_slots + 1, *shape] tensors, one per run
+that asks for it; the last row (`idle_slot`) belongs to no request: the idle lanes of a
+captured decode batch point there, so whatever a part writes for them lands nowhere.
 """
 
 from __future__ import annotations
@@ -50,7 +51,7 @@ class LayerCache:
     num_pages: int
     k_pages: torch.Tensor | None   # [num_pages, nkv, P, hd]
     v_pages: torch.Tensor | None   # [num_pages, nkv, hd, P]
-    state: torch.Tensor | None = None   # [num_slots, *shape] for fixed-size state
+    state: torch.Tensor | None = None   # [num_slots + 1, *shape] for fixed-size state
 
 
 class CacheStorage:
@@ -65,6 +66,9 @@ class CacheStorage:
                 len(g.runs), n, g.num_kv_heads, page_size, g.head_dim, dtype=dtype, device=device))
             self.v_tensors.append(torch.zeros(
                 len(g.runs), n, g.num_kv_heads, g.head_dim, page_size, dtype=dtype, device=device))
+        self.idle_slot = num_slots
+        self.state_runs = tuple(r for r, need in enumerate(needs)
+                                if isinstance(need, SlotStateNeed))
         self.views: list[LayerCache | None] = []
         for r, need in enumerate(needs):
             if isinstance(need, PagedKVNeed):
@@ -73,7 +77,7 @@ class CacheStorage:
                 self.views.append(LayerCache(g, page_size, counts[g], self.k_tensors[g][i],
                                              self.v_tensors[g][i]))
             elif isinstance(need, SlotStateNeed):
-                state = torch.zeros(num_slots, *need.shape, dtype=need.dtype, device=device)
+                state = torch.zeros(num_slots + 1, *need.shape, dtype=need.dtype, device=device)
                 self.views.append(LayerCache(-1, page_size, 0, None, None, state))
             else:
                 self.views.append(None)

@@ -47,6 +47,7 @@ class Config:
     dtype: torch.dtype = torch.bfloat16
     seed: int = 0
     enable_prefix_caching: bool = False   # share cached full pages between equal prefixes
+    warmup: bool = True                   # largest dummy step and graph capture at construction
 
     def __post_init__(self) -> None:
         if not os.path.isdir(self.model):

@@ -71,11 +71,12 @@ class StaticDecodeBatch:
 
     `fill` rewrites the contents for the step's entries; lanes beyond them are idle:
     token 0 at position 0 with no pages, so they write nothing to the cache
-    (as the reference pads with slot -1, engine/generation/model_runner.py:253-276).
+    (as the reference pads with slot -1, engine/generation/model_runner.py:253-276),
+    and with state slot `idle_slot`, which no request owns.
     """
 
-    def __init__(self, device, bucket: int, widths: list[int]) -> None:
-        self.bucket, self.widths = bucket, widths
+    def __init__(self, device, bucket: int, widths: list[int], idle_slot: int = 0) -> None:
+        self.bucket, self.widths, self.idle_slot = bucket, widths, idle_slot
         self.offs, total = decode_layout(bucket, widths)
         self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
         self.dev = torch.zeros(total, dtype=torch.int32, device=device)
@@ -108,12 +109,20 @@ class StaticDecodeBatch:
 
     def fill(self, entries, temperatures=None, keys=None) -> None:
         o, B, n = self.offs, self.bucket, len(entries)
+        if n > B:
+            raise ValueError(f"{n} entries for a static batch of {B} lanes")
+        for e in entries:
+            for t, w in zip(e.cache.tables, self.widths):
+                if len(t) > w:
+                    raise ValueError(
+                        f"request {e.cache.request_id!r}: block table of {len(t)} pages "
+                        f"is wider than the static batch's {w}")
         self.copied.synchronize()          # the last copy out of the pinned buffer is done
         h = self.host.numpy()
         h[o[0] + n:o[0] + B] = 0
         h[o[1] + n:o[1] + B] = 0
         h[o[4] + n:o[4] + B] = 1
-        h[o[5] + n:o[5] + B] = 0
+        h[o[5] + n:o[5] + B] = self.idle_slot
         starts = [e.start for e in entries]
         h[o[0]:o[0] + n] = [e.tokens[0] for e in entries]
         h[o[1]:o[1] + n] = starts

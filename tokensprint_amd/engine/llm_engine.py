@@ -30,16 +30,23 @@ class LLMEngine:
         if model.ctx.dtype != config.dtype:
             raise ValueError(f"model runs in {model.ctx.dtype}, config asks for {config.dtype}")
         page = config.kvcache_block_size
+        on_gpu = model.ctx.device.type == "cuda"
+        graph_len = None if config.enforce_eager or not on_gpu else config.max_model_len
         num_pages = config.num_kvcache_blocks
         if num_pages < 0:
-            num_pages = self._pages_from_free_memory(model, config)
+            num_pages = self._pages_from_free_memory(model, config, graph_len)
             config.num_kvcache_blocks = num_pages
         self.runner = ModelRunner(
             model, page_size=page, num_pages=num_pages, num_slots=config.max_num_seqs,
-            graph_max_len=None if config.enforce_eager or model.ctx.device.type != "cuda"
-            else config.max_model_len)
+            graph_max_len=graph_len)
         if config.enable_prefix_caching:
             self.runner.manager.enable_prefix_cache()
+        if config.warmup and on_gpu:
+            # before the first request: kernels loaded, the library's choices made, every
+            # decode bucket captured (engine/generation/model_runner.py:28-35 warms up and
+            # captures in its constructor)
+            self.runner.dummy_step(*self.largest_step(config))
+            self.runner.capture_all()
         self.scheduler = Scheduler(
             self.runner.manager, max_num_batched_tokens=config.max_num_batched_tokens,
             max_num_seqs=config.max_num_seqs, max_model_len=config.max_model_len,
@@ -49,18 +56,59 @@ class LLMEngine:
         self.requests: dict[int, Request] = {}
 
     @staticmethod
-    def _pages_from_free_memory(model: Model, config: Config) -> int:
-        """free * utilization minus room for one step's activations, in pages
+    def largest_step(config: Config) -> tuple[int, int]:
+        """(tokens, requests) of the largest step the scheduler can put together: the
+        token budget, or, when prefill is not chunked, a recomputed request of
+        max_model_len - 1 tokens alone; as many requests as may be live, since each can
+        ask for a row of logits."""
+        tokens = config.max_num_batched_tokens
+        if not config.chunked_prefill:
+            tokens = max(tokens, config.max_model_len - 1)
+        fewest = -(-tokens // (config.max_model_len - 1))
+        return tokens, max(fewest, min(config.max_num_seqs, tokens))
+
+    @staticmethod
+    def measure_step_memory(model: Model, config: Config, graph_len) -> int:
+        """Device bytes the engine needs beside weights and cache: the peak of its largest
+        step plus what the captured decode graphs keep, measured on a throw-away cache
+        just large enough for that step (the reference measures its dummy forward's peak
+        the same way, engine/generation/model_runner.py:288-308,392-398)."""
+        import gc
+        device = model.ctx.device
+        tokens, requests = LLMEngine.largest_step(config)
+        page = config.kvcache_block_size
+        torch.cuda.synchronize(device)
+        torch.cuda.empty_cache()
+        probe = ModelRunner(model, page_size=page, num_pages=-(-tokens // page) + requests,
+                            num_slots=config.max_num_seqs, graph_max_len=graph_len)
+        torch.cuda.synchronize(device)
+        before = torch.cuda.memory_reserved(device)
+        torch.cuda.reset_peak_memory_stats(device)
+        probe.dummy_step(tokens, requests)
+        step_peak = torch.cuda.max_memory_reserved(device) - before
+        torch.cuda.empty_cache()
+        before = torch.cuda.memory_reserved(device)
+        probe.capture_all()
+        torch.cuda.synchronize(device)
+        torch.cuda.empty_cache()
+        graphs = torch.cuda.memory_reserved(device) - before
+        del probe
+        gc.collect()
+        torch.cuda.empty_cache()
+        log.info("largest step (%d tokens, %d requests) peaks at %.1f MiB; captured graphs "
+                 "keep %.1f MiB", tokens, requests, step_peak / 2**20, graphs / 2**20)
+        return max(step_peak, 0) + max(graphs, 0)
+
+    @staticmethod
+    def _pages_from_free_memory(model: Model, config: Config, graph_len=None) -> int:
+        """free * utilization minus the measured needs of the steps, in pages
         (engine/generation/model_runner.py:392-411)."""
         device = model.ctx.device
         if device.type != "cuda":
             raise ValueError("num_kvcache_blocks must be given when there is no GPU to size from")
+        steps = LLMEngine.measure_step_memory(model, config, graph_len)
         free, _ = torch.cuda.mem_get_info(device)
-        spec = model.spec
-        widest = max(spec.width * 8, spec.vocab_size // 8)
-        act = config.max_num_batched_tokens * widest * 4 * 4
-        logits = min(config.max_num_seqs, config.max_num_batched_tokens) * spec.vocab_size * 4 * 2
-        available = free * config.gpu_memory_utilization - act - logits
+        available = free * config.gpu_memory_utilization - steps
         pages = ModelRunner.pages_that_fit(model, config.kvcache_block_size, int(available),
                                            config.dtype)
         # no request can use more than max_model_len tokens
@@ -68,7 +116,9 @@ class LLMEngine:
         pages = min(pages, cap)
         if pages < 1:
             raise RuntimeError("Insufficient GPU memory for the key/value cache: "
-                               f"available={int(available)} bytes")
+                               f"available={int(available)} bytes after {steps} bytes for the "
+                               "steps themselves")
+        log.info("key/value cache: %d pages of %d tokens", pages, config.kvcache_block_size)
         return pages
 
     # ------------------------------------------------------------ requests

@@ -28,16 +28,23 @@ class ModelRunner:
         needs = model.cache_needs()
         self.storage = CacheStorage(needs, page_size, num_pages, num_slots,
                                     cache_dtype or self.dtype, self.device)
-        self.manager = CacheManager(self.storage.groups, page_size, num_pages, num_slots)
+        self.manager = CacheManager(self.storage.groups, page_size, num_pages, num_slots,
+                                    state_runs=self.storage.state_runs)
         self.builder = BatchBuilder(self.device, len(self.storage.groups),
                                     vocab_size=model.spec.vocab_size,
                                     max_position=model.spec.max_position)
         self.page_size = page_size
+        self.num_slots = num_slots
         self.graph_max_len = graph_max_len
-        self.graphs: dict[int, tuple] = {}      # bucket -> (graph, static batch, logits)
+        self.graphs: dict[int, tuple] = {}      # bucket -> (graph, static batch, logits, tokens)
+        self._graph_pool = None                 # one memory pool for every captured bucket
+        # a part that cannot be captured (it says so) keeps every step eager
+        capture = bool(graph_max_len) and self.device.type == "cuda" and model.all_capturable()
         top = min(graph_max_batch, num_slots)
         self.buckets = sorted({b for b in [1, 2, 4, 8] + list(range(16, top + 1, 16)) + [top]
-                               if b <= top}) if graph_max_len else []
+                               if b <= top}) if capture else []
+        self._graph_widths = [-(-graph_max_len // page_size)] * len(self.storage.groups) \
+            if capture else []
 
     @staticmethod
     def pages_that_fit(model: Model, page_size: int, free_bytes: int,
@@ -73,11 +80,15 @@ class ModelRunner:
         for e in entries:
             if len(e.tokens) != 1 or e.want != [0] or e.start + 1 > self.graph_max_len:
                 return None
+            # a cache extended beyond what the captured block tables can name (a caller
+            # may reserve ahead) is served eagerly
+            if any(len(t) > w for t, w in zip(e.cache.tables, self._graph_widths)):
+                return None
         return next(b for b in self.buckets if b >= len(entries))
 
     def _capture(self, bucket: int):
-        widths = [-(-self.graph_max_len // self.page_size)] * len(self.storage.groups)
-        static = StaticDecodeBatch(self.device, bucket, widths)
+        static = StaticDecodeBatch(self.device, bucket, self._graph_widths,
+                                   idle_slot=self.storage.idle_slot)
         static.batch.max_ctx_len = self.graph_max_len
         static.fill([])
         torch.cuda.synchronize(self.device)
@@ -88,12 +99,51 @@ class ModelRunner:
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, pool=self._graph_pool):
             logits = self.run(static.batch)
             # the draw is part of the captured step: rows with temperature 0 are greedy
             tokens = self.model.ctx.ops.sample(logits, static.temperatures, static.keys)
+        if self._graph_pool is None:
+            self._graph_pool = graph.pool()
         self.graphs[bucket] = (graph, static, logits, tokens)
         return self.graphs[bucket]
+
+    def capture_all(self) -> None:
+        """Capture every decode bucket now, the largest first so that the smaller ones fit
+        into the memory it took (engine/generation/model_runner.py:334,373-379 captures in
+        that order for that reason).  Without this a bucket is captured at its first use."""
+        for bucket in reversed(self.buckets):
+            if bucket not in self.graphs:
+                self._capture(bucket)
+
+    def dummy_step(self, num_tokens: int, num_entries: int) -> int:
+        """Run one step of `num_tokens` zero tokens in `num_entries` requests (fewer of
+        either if the pool or the slots do not hold as many), each asking for its last
+        token's logits, and give everything back: loads the kernels, lets the library
+        choose its algorithms and shows what such a step costs in memory.  Returns the
+        tokens it ran."""
+        manager = self.manager
+        if manager.live:
+            raise RuntimeError("a dummy step needs an engine without live requests")
+        n = max(1, min(num_entries, manager.slots.num_free, num_tokens))
+        pool = min(p.num_free for p in manager.pools) if manager.pools else num_tokens
+        longest = self.model.spec.max_position
+        per = max(1, min(num_tokens // n, longest, (pool // n) * self.page_size))
+        if manager.pools and pool < n:
+            n, per = max(1, pool), min(self.page_size, longest)
+        entries = []
+        for i in range(n):
+            rc = manager.admit(("dummy", i))
+            manager.extend(rc, per)
+            entries.append(StepEntry(rc, [0] * per, 0, [per - 1]))
+        try:
+            self.run(self.build(entries))
+            if self.device.type == "cuda":
+                torch.cuda.synchronize(self.device)
+        finally:
+            for e in entries:
+                manager.free(e.cache)
+        return n * per
 
     def decode_and_sample(self, entries: list[StepEntry], temperatures, keys):
         """One decode step with the draw inside the captured graph: token ids (int32 device

@@ -1,5 +1,8 @@
 """What travels between the product that ends a sub-layer and the norm and product that
-follow it, when a kernel provider fuses the residual add and the norm into the two."""
+follow it, when a kernel provider fuses the residual add and the norm into the two, and
+the optional mixins through which parts take part in that.  The part interfaces
+(tokensprint_amd.parts.base) know none of this: a part that uses neither mixin works
+between parts that do."""
 
 from __future__ import annotations
 
@@ -31,3 +34,33 @@ class PreparedRows:
     rows: torch.Tensor
     sumsq: torch.Tensor
     hint: NormHint
+
+
+def fused_rmsnorm_of(norm):
+    """(weight, eps) if `norm` says it is a plain RMSNorm that a kernel may fuse into the
+    product after it (it has a `fused_rmsnorm()` that returns them), else None."""
+    probe = getattr(norm, "fused_rmsnorm", None)
+    return probe() if callable(probe) else None
+
+
+class StreamProducts:
+    """Mixin for a part (with `.ops` and `.ctx`) whose first product may take the residual
+    add and RMSNorm before it, and whose last product may add itself into the stream."""
+
+    def first_product_hint(self, norm, weight: torch.Tensor, silu_mul: bool = False):
+        """For `stream_hint`: the hint, if `norm` can be fused and the provider has the
+        kernels, else None."""
+        fused = fused_rmsnorm_of(norm)
+        if fused is None or not hasattr(self.ops, "linear_into_stream"):
+            return None
+        return NormHint(fused[0], fused[1], weight, silu_mul)
+
+    def last_product(self, x: torch.Tensor, weight: torch.Tensor, resid: torch.Tensor, hint):
+        """The product that ends a sub-layer: x W^T as the stream's next delta, or, where
+        `hint` (a NormHint) says what follows and the provider can, added into `resid` at
+        once and handed on as PreparedRows (which stand in delta's place)."""
+        if isinstance(hint, NormHint):
+            prepared = self.ops.linear_into_stream(x, weight, resid, hint)
+            if prepared is not None:
+                return prepared
+        return self.ops.linear(x, weight, self.ctx.dtype)

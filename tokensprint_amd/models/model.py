@@ -96,10 +96,19 @@ class Model:
         else:
             resid_rows = ops.gather_rows(resid, batch.logit_rows)
             delta_rows = None if delta is None else ops.gather_rows(delta, batch.logit_rows)
-        fused = self.final_norm.fused_rmsnorm()
-        if fused is not None:
-            return ops.norm_linear(resid_rows, delta_rows, fused[0], fused[1], self.head.weight,
-                                   torch.float32)[0]
-        h = self.final_norm.forward(resid_rows) if delta_rows is None \
-            else self.final_norm.add_forward(resid_rows, delta_rows)
-        return self.head.forward(h)
+        return self.head.forward_from_stream(resid_rows, delta_rows, self.final_norm)
+
+    # ------------------------------------------------------------ accounting
+    def step_weight_bytes(self) -> int:
+        """Bytes of every tensor a step reads whole, each counted once (a tied head and
+        the embedding share one table): the weight traffic of a decode step."""
+        seen, total = set(), 0
+        for part in self.parts():
+            for t in part.step_read_tensors():
+                if t.data_ptr() not in seen:
+                    seen.add(t.data_ptr())
+                    total += t.numel() * t.element_size()
+        return total
+
+    def all_capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())

@@ -50,7 +50,7 @@ def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
         order=tuple(Run(i) for i in range(cfg.num_layers)),
         final_norm=PartSpec("rmsnorm", {
             "dim": cfg.hidden_size, "eps": cfg.rms_norm_eps, "weight": "model.norm.weight"}),
-        head=head, max_position=cfg.max_position,
+        head=head, max_position=cfg.max_position, eos_token_id=cfg.eos_token_id,
     )
 
 

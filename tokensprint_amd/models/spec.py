@@ -54,6 +54,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_position: int
+    eos_token_id: int | None = None       # the checkpoint's end-of-sequence token, if it names one
 
     def validate(self) -> None:
         if not self.order:

@@ -12,11 +12,12 @@ from __future__ import annotations
 
 import torch
 
+from tokensprint_amd.kernels.stream import StreamProducts, fused_rmsnorm_of
 from tokensprint_amd.parts.base import MIXERS, Mixer, PagedKVNeed, TensorDecl, register
 
 
 @register(MIXERS, "gqa_attention")
-class GroupedQueryAttention(Mixer):
+class GroupedQueryAttention(StreamProducts, Mixer):
     """params: prefix, num_heads, num_kv_heads, head_dim, qk_norm (bool), qk_norm_eps,
     position (name of a shared position encoding or None), window (None = all keys),
     own_kv (False: the layer has no k/v weights and only reads another run's cache).
@@ -72,7 +73,7 @@ class GroupedQueryAttention(Mixer):
         return self.first_product_hint(norm, self.w_qkv)
 
     def forward_from_stream(self, resid, delta, norm, batch, cache, write_cache, hint=None):
-        fused = norm.fused_rmsnorm()
+        fused = fused_rmsnorm_of(norm)
         if fused is None:
             return super().forward_from_stream(resid, delta, norm, batch, cache, write_cache)
         qkv, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_qkv,

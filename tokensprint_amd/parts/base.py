@@ -18,9 +18,6 @@ from typing import Any, Callable
 
 import torch
 
-from tokensprint_amd.kernels.stream import NormHint
-
-
 # ------------------------------------------------------------------ declarations
 
 
@@ -81,32 +78,29 @@ class Part:
     def load(self, get: Callable[[str], torch.Tensor | None]) -> None:
         """Take the declared tensors (`get(name)`, None if optional and absent)."""
 
-    # -- the residual add and norm split over the product before and the product after
-    def first_product_hint(self, norm: "Norm", weight: torch.Tensor, silu_mul: bool = False):
-        """For `stream_hint` of a part whose first product is `weight` after `norm`: the
-        hint, if the norm is one a kernel may fuse and the provider has such kernels."""
-        fused = norm.fused_rmsnorm()
-        if fused is None or not hasattr(self.ops, "linear_into_stream"):
-            return None
-        return NormHint(fused[0], fused[1], weight, silu_mul)
+    #: False for a part that cannot run inside a captured graph (it synchronises with the
+    #: host, or its work depends on values the host reads from the device).  A decode step
+    #: of a model with such a part always runs eagerly.  A part that leaves this True must,
+    #: in a decode step, use only the batch's device tensors: the host lists of a captured
+    #: batch (`q_lens`, `starts`) are placeholders.
+    capturable = True
 
-    def last_product(self, x: torch.Tensor, weight: torch.Tensor, resid: torch.Tensor, hint):
-        """The product that ends a sub-layer: x W^T as the stream's next delta, or, where
-        `hint` says what follows and the provider can, added into `resid` at once and
-        handed on as prepared rows (which stand in delta's place)."""
-        if hint is not None:
-            prepared = self.ops.linear_into_stream(x, weight, resid, hint)
-            if prepared is not None:
-                return prepared
-        return self.ops.linear(x, weight, self.ctx.dtype)
+    def held_tensors(self) -> list[torch.Tensor]:
+        """Every tensor this part keeps on the device (weights taken in `load`, tables)."""
+        out = []
+        for value in vars(self).values():
+            for t in value if isinstance(value, (list, tuple)) else (value,):
+                if isinstance(t, torch.Tensor):
+                    out.append(t)
+        return out
+
+    def step_read_tensors(self) -> list[torch.Tensor]:
+        """The tensors a step reads whole, whatever its tokens are: what a decode step's
+        memory traffic is counted from.  Default: everything held."""
+        return self.held_tensors()
 
 
 class Norm(Part):
-    def fused_rmsnorm(self):
-        """(weight, eps) if this norm is a plain RMSNorm a kernel may fuse into the product
-        that follows it, else None."""
-        return None
-
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """Normalised copy of x [T, width] in the activation dtype."""
         raise NotImplementedError
@@ -140,8 +134,10 @@ class Mixer(Part):
         raise NotImplementedError
 
     def stream_hint(self, norm: Norm):
-        """A NormHint if this part, reading the stream through `norm`, takes prepared
-        rows in `delta`'s place (see `Part.last_product`), else None."""
+        """What this part lets the producer of the stream know about its first product
+        behind `norm`, or None.  Whatever it returns comes back as `hint` to the part
+        that runs before it; the kernel provider's fused forms define the one kind there
+        is (tokensprint_amd.kernels.stream), and a part may ignore all of it."""
         return None
 
     def forward_from_stream(self, resid, delta, norm: Norm, batch, cache, write_cache: bool,
@@ -174,8 +170,8 @@ class Block:
     The stream travels as (resid, delta): resid is float32 [T, width]; delta is
     the last sub-layer's output not yet added (None at the very start), so the
     add can be fused into the next norm.  Where the part that reads the stream next
-    gives a `stream_hint`, the part before it may hand on prepared rows instead of a
-    delta (`Part.last_product`); only that reader ever sees them.
+    gives a `stream_hint`, the part before it may hand on, instead of a delta, whatever
+    that hint's protocol defines; only that reader ever sees it.
     """
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,

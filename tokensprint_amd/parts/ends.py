@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import torch
 
+from tokensprint_amd.kernels.stream import fused_rmsnorm_of
 from tokensprint_amd.parts.base import Part, TensorDecl
 
 
@@ -30,6 +31,9 @@ class Embedding(Part):
 
     def forward(self, token_ids):
         return self.ops.embed(self.table, token_ids)
+
+    def step_read_tensors(self):
+        return []          # a step reads the rows of its tokens, not the table
 
 
 class Head(Part):
@@ -54,3 +58,14 @@ class Head(Part):
 
     def forward(self, h):
         return self.ops.linear(h, self.weight, torch.float32)
+
+    def forward_from_stream(self, resid, delta, norm):
+        """Logits of the rows of the residual stream (resid float32, delta the last
+        sub-layer's output not yet added, or None) behind `norm`; the add and the norm go
+        into the product where the norm and the kernel provider allow it."""
+        fused = fused_rmsnorm_of(norm)
+        if fused is not None:
+            return self.ops.norm_linear(resid, delta, fused[0], fused[1], self.weight,
+                                        torch.float32)[0]
+        h = norm.forward(resid) if delta is None else norm.add_forward(resid, delta)
+        return self.forward(h)

@@ -7,11 +7,12 @@ from __future__ import annotations
 
 import torch
 
+from tokensprint_amd.kernels.stream import StreamProducts, fused_rmsnorm_of
 from tokensprint_amd.parts.base import FEED_FORWARDS, FeedForward, TensorDecl, register
 
 
 @register(FEED_FORWARDS, "swiglu")
-class SwiGLU(FeedForward):
+class SwiGLU(StreamProducts, FeedForward):
     """params: prefix, inner_dim."""
 
     def __init__(self, params, ctx):
@@ -38,7 +39,7 @@ class SwiGLU(FeedForward):
         return self.first_product_hint(norm, self.w_gate_up, silu_mul=True)
 
     def forward_from_stream(self, resid, delta, norm, batch, hint=None):
-        fused = norm.fused_rmsnorm()
+        fused = fused_rmsnorm_of(norm)
         if fused is None:
             return super().forward_from_stream(resid, delta, norm, batch)
         act, resid = self.ops.norm_linear(resid, delta, fused[0], fused[1], self.w_gate_up,

@@ -33,6 +33,9 @@ class RotaryEncoding(PositionEncoding):
     def rotary_tables(self):
         return self.cos, self.sin
 
+    def step_read_tensors(self):
+        return []          # a step reads the rows of its positions, not the tables
+
     def apply(self, q, k, positions):
         self.ops.rope_inplace(q, positions, self.cos, self.sin)
         if k is not None:
