@@ -137,7 +137,9 @@ def test_captured_decode_steps_with_many_requests(setup):
         assert runner._graph_bucket(entries) == 20
         logits = runner.step(entries).clone()
         for (rc, pos), row in zip(live, logits):
-            torch.testing.assert_close(row.cpu(), ref["r3"][pos], rtol=rtol, atol=atol)
+            want = ref["r3"][pos]
+            assert ((row.cpu() - want).abs() <= drives.row_tolerance(ref["r3"], rtol, atol)[pos]).all(), \
+                f"step {step}, position {pos}: {(row.cpu() - want).abs().max():.3e}"
         for item in live:
             item[1] += 1
         if step % 2 == 0:                     # eager work between replays

@@ -193,6 +193,11 @@ class ToyTop1FeedForward(FeedForward):
 
     def forward(self, h, batch):
         pick = (h.float() @ self.router.float().T).argmax(-1)
+        if batch.max_q_len == 1:
+            # a decode step may be captured: no row lists on the host, both experts run
+            # and each token keeps its own
+            both = [self.ops.linear(h, e, h.dtype) for e in self.e]
+            return torch.where((pick == 0)[:, None], both[0], both[1])
         out = torch.zeros_like(h)
         for i in (0, 1):
             rows = (pick == i).nonzero().squeeze(-1)
