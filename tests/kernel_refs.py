@@ -116,12 +116,14 @@ class TorchOps:
 
     # ---------------------------------------------------------------- attention
     def paged_attention(self, q, batch, table, cache, *, num_heads, num_kv_heads, head_dim,
-                        scale, window):
+                        scale, window, only=None):
+        """`only`: compute just these flat tokens (a test's choice; the other rows of the
+        result are left unset)."""
         T = q.shape[0]
         P = cache.page_size
         group = num_heads // num_kv_heads
         out = torch.empty(T, num_heads, head_dim, dtype=torch.float32, device=q.device)
-        for t in range(T):
+        for t in (range(T) if only is None else only):
             b = int(batch.entry_of_token[t])
             p = int(batch.positions[t])
             lo = 0 if window is None else max(0, p - window + 1)

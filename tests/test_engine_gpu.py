@@ -180,3 +180,51 @@ def test_eps_of_the_per_head_norms_shows(name, dtype, tmp_path, gpu_device):
     assert (other - ref["a"]).abs().max() > margin * (atol + rtol * ref["a"].abs().max())
     col = drives.drive_prefill_then_decode(runner_for(model, page, 128 // page), requests, tail=12)
     drives.compare(col, ref, rtol, atol)
+
+
+@pytest.fixture(scope="module")
+def wide_bfloat16(tmp_path_factory, gpu_device):
+    cfg, seed, page = GPU_ONLY["F"]
+    d = tmp_path_factory.mktemp("wideF")
+    write_random_model(d, cfg, seed, torch.bfloat16)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, torch.bfloat16, gpu_device)
+    tokens = random_prompt(48, cfg["vocab_size"], 300)
+    return model, page, tokens, plain.forward_logits(pcfg, w, tokens)
+
+
+@pytest.mark.parametrize("captured", [False, True], ids=["eager", "captured"])
+@pytest.mark.parametrize("lanes", [4, 5, 8, 9, 16, 17, 64, 65])
+def test_decode_lanes_on_both_sides_of_each_kernel_choice(wide_bfloat16, lanes, captured):
+    """Which kernel serves a product depends on the number of rows: the output head goes
+    to the library from 5 rows, the layer products of this width from 9, those with a
+    short K from 17, everything from 65.  A decode step with one lane fewer and one lane
+    more than each of these must give the plain logits, eagerly and from a captured graph."""
+    from tokensprint_amd.engine import StepEntry
+    model, page, tokens, ref = wide_bfloat16
+    rtol, atol = TOL[torch.bfloat16]
+    runner = ModelRunner(model, page_size=page, num_pages=lanes * (64 // page + 1),
+                         num_slots=lanes, graph_max_len=64 if captured else None,
+                         graph_max_batch=lanes)
+    live = []
+    for i in range(lanes):
+        rc = runner.manager.admit(i)
+        head = 8 + i % 30
+        runner.manager.extend(rc, head)
+        live.append([rc, head])
+    # the prompts' heads, several requests a step
+    for first in range(0, lanes, 16):
+        runner.step([StepEntry(rc, tokens[:head], 0, []) for rc, head in live[first:first + 16]])
+    for step in range(3):
+        entries = []
+        for rc, pos in live:
+            runner.manager.extend(rc, pos + 1)
+            entries.append(StepEntry(rc, tokens[pos:pos + 1], pos, [0]))
+        assert (runner._graph_bucket(entries) is not None) == captured
+        logits = runner.step(entries).float().cpu()
+        bound = drives.row_tolerance(ref, rtol, atol)
+        for (rc, pos), row in zip(live, logits):
+            assert ((row - ref[pos]).abs() <= bound[pos]).all(), \
+                f"{lanes} lanes, step {step}, position {pos}: {(row - ref[pos]).abs().max():.3e}"
+        for item in live:
+            item[1] += 1

@@ -604,6 +604,80 @@ def test_attend_finds_one_far_key_in_a_decode_step(ops, gpu_device, ctx):
             torch.testing.assert_close(out[0, kvh * 2].float(), want[kvh], rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lo", [512, 528, 544, 531, 700])
+def test_window_edge_in_a_decode_step(ops, gpu_device, dtype, lo):
+    """A window's lower edge, with a key made to dominate on either side of it: the key
+    at p-W+1 must be found (the output is its value row) and the key at p-W ignored.  The
+    edge is put on a 128-key chunk's, a page's and a 32-key block's first key, inside a
+    block, and on the step's own key (W = 1).  With random keys alone one key more or
+    less moves a row by about 1/W, which a tolerance hides."""
+    nq, nkv, hd, page, ctx = 4, 2, 128, 16, 700
+    W = ctx + 1 - lo                       # the query is at position ctx
+    kw = dict(num_heads=nq, num_kv_heads=nkv, kv_in_row=nkv, head_dim=hd, q_weight=None,
+              k_weight=None, eps=0.0, cos_sin=None, scale=1.0, window=W)
+    for planted in (lo - 1, lo):
+        batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                                spans=[(ctx, 1)], seed=23)
+        qkv = rand((1, (nq + 2 * nkv) * hd), dtype, gpu_device, 24)
+        row = qkv.view(nq + 2 * nkv, hd)
+        if planted == ctx:                 # the step's own key
+            for kvh in range(nkv):
+                row[nq + kvh] = (4.0 * row[kvh * 2].float()).to(dtype)
+            value = [row[nq + nkv + kvh].float() for kvh in range(nkv)]
+        else:
+            phys = int(table[0, planted // page])
+            for kvh in range(nkv):
+                cache.k_pages[phys, kvh, planted % page] = (4.0 * row[kvh * 2].float()).to(dtype)
+            value = [cache.v_pages[phys, kvh, :, planted % page].float() for kvh in range(nkv)]
+        theirs = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                             cache.k_pages.clone(), cache.v_pages.clone())
+        out = ops.attend(qkv, batch, table, cache, True, **kw).view(1, nq, hd).float()
+        ref = REF.attend(qkv, batch, table, theirs, True, **kw).view(1, nq, hd).float()
+        torch.testing.assert_close(out, ref, rtol=2e-2, atol=2e-2)
+        for kvh in range(nkv):
+            if planted == lo:
+                torch.testing.assert_close(out[0, kvh * 2], value[kvh], rtol=2e-2, atol=2e-2)
+            else:
+                assert (out[0, kvh * 2] - value[kvh]).abs().max() > 0.5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("start,n,picks", [(683, 2, [0]), (619, 2, [0]), (603, 2, [0]), (601, 2, [0]),
+                                           (600, 2200, [0, 3, 19, 83, 1000, 2198])])
+def test_window_edge_in_portions(ops, gpu_device, dtype, start, n, picks):
+    """The same for portions of prompts, through `paged_attention`: two tokens (each query
+    has an edge of its own, one key apart) and a portion long enough for the kernels in
+    which a wavefront walks several query tiles.  For a picked query at position p the
+    key at p-W+1, its window's first, is aligned with the first head of each group, and
+    the next token gets the same query vector: the picked query's output is that key's
+    value row, the next token's, one position on, is not; both equal the plain reference.
+    The edges fall on a chunk's, a block's and a page's first key and between."""
+    nq, nkv, hd, page, W = 16, 8, 128, 16, 300
+    if dtype == torch.float32 and n > 2:
+        pytest.skip("the long-portion kernels are bfloat16 only; float32 takes the general one")
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=[(start, n)], seed=31)
+    q = rand((n, nq, hd), dtype, gpu_device, 32)
+    group = nq // nkv
+    value = {}
+    for i in picks:
+        where = start + i - W + 1
+        q[i + 1] = q[i]
+        phys = int(table[0, where // page])
+        for kvh in range(nkv):
+            cache.k_pages[phys, kvh, where % page] = (4.0 * q[i, kvh * group].float()).to(dtype)
+            value[(i, kvh * group)] = cache.v_pages[phys, kvh, :, where % page].float()
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=1.0, window=W)
+    out = ops.paged_attention(q, batch, table, cache, **kw).float()
+    rows = sorted(picks + [i + 1 for i in picks])
+    ref = REF.paged_attention(q, batch, table, cache, only=rows, **kw).float()
+    torch.testing.assert_close(out[rows], ref[rows], rtol=2e-2, atol=2e-2)
+    for (i, head), row in value.items():
+        torch.testing.assert_close(out[i, head], row, rtol=2e-2, atol=2e-2)
+        assert (out[i + 1, head] - row).abs().max() > 0.5, (i, head)
+
+
 def test_argmax_and_ties(ops, gpu_device):
     logits = rand((9, 151936), torch.float32, gpu_device, 30)
     assert torch.equal(ops.argmax(logits).long(), logits.argmax(-1))

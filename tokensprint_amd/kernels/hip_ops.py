@@ -176,8 +176,12 @@ class HipOps:
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
         if self._library_ok(x, weight):
-            out = torch.matmul(x, weight.t())
-            return out if out_dtype == torch.bfloat16 else out.float()
+            if out_dtype == torch.bfloat16:
+                return torch.matmul(x, weight.t())
+            # the library's float32 sums leave as they are (the output head's logits):
+            # not rounded to bfloat16 and widened, so that logits are of one precision
+            # on both sides of the row count at which the library takes over
+            return torch.mm(x, weight.t(), out_dtype=torch.float32)
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         if self._mfma_ok(x, weight):
             self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
@@ -198,8 +202,8 @@ class HipOps:
     # At the layer shapes of the 8B and 32B models (weights above 2^23 elements, products
     # bound by bandwidth, not latency) every workgroup's reading of the rows of x costs
     # as much as the weights from 16 rows on, and the library is ahead from 9 rows.
-    # Its result is bfloat16 (float32 accumulation), as the reference's logits are;
-    # float32 results of such a product are that result widened.
+    # It accumulates in float32 and stores the type asked for: bfloat16 activations, and
+    # float32 logits at the output head (the reference's logits are bfloat16).
     LIBRARY_ROWS = 65
     LIBRARY_ROWS_WIDE = 17
     LIBRARY_ROWS_HEAD = 5
