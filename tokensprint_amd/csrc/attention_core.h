@@ -178,7 +178,11 @@ __device__ __forceinline__ void load_query(TileState<HD>& t, const bf16_t* qrow,
 // (a wave-uniform branch).  Far into a long context most blocks bring none.  For kernels
 // whose loads of the next block are in flight across this call the branch costs more
 // than it saves (the waits at its join are for all of them).
-template <int HD, bool LAZY = false>
+//
+// PERM: the keys of the block are assigned to the rows of the two score products so that
+// lane (r, g) holds the scores of keys g * 8 .. g * 8 + 7 (row i of product b is key
+// (i / 4) * 8 + b * 4 + i % 4) instead of keys g * 4 .. + 3 of each 16-key half.
+template <int HD, bool LAZY = false, bool PERM = false>
 __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>& b, int kb,
                                             float scale_log2, bool interior, int g) {
   constexpr int KS = TileState<HD>::KS, DB = TileState<HD>::DB;
@@ -196,7 +200,7 @@ __device__ __forceinline__ void tile_update(TileState<HD>& t, const KvBlock<HD>&
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = kb + blk * 16 + g * 4 + i;
+        const int key = PERM ? kb + g * 8 + blk * 4 + i : kb + blk * 16 + g * 4 + i;
         st[blk][i] = (key <= t.pos && key >= t.lo) ? st[blk][i] : -INFINITY;
       }
   }

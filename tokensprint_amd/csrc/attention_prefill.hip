@@ -1,5 +1,7 @@
 // Paged causal attention on the matrix cores for long portions of prompts (bfloat16).
 //
+// The tile list comes sorted by the length of the key range, longest first.
+//
 // A wavefront works on TPW consecutive 16-row query tiles of one batch entry and walks
 // their common key range alone, 32 keys at a time, with the next block's keys and values
 // in flight while the current block is worked on.  Every K and V block it loads serves
@@ -21,7 +23,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(AttentionMfmaArg
   const int head_slot = blockIdx.x % heads;
   const int tile_rank = (blockIdx.x / heads) * 4 + wave;
   if (tile_rank >= args.num_tiles) return;
-  const int tile = args.num_tiles - 1 - tile_rank;
+  const int tile = tile_rank;                                // the list is sorted: longest first
   const int kvh = head_slot / args.head_blocks;
   const int hb = head_slot % args.head_blocks;
   const int entry = uniform(args.tiles[tile * 3]), tok0 = uniform(args.tiles[tile * 3 + 1]),
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
   // items with the longest key ranges, longest first, the second half the shortest,
   // shortest first, so a unit's workgroups add up to about the same work.
   const int rank = blockIdx.x / heads, half = (args.num_tiles + 1) / 2;
-  const int item = rank < half ? args.num_tiles - 1 - rank : rank - half;
+  const int item = rank < half ? rank : args.num_tiles - 1 - (rank - half);   // sorted: longest first
   const int kvh = head_slot / args.head_blocks;
   const int hb = head_slot % args.head_blocks;
   const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
@@ -305,6 +307,184 @@ __global__ __launch_bounds__(256, HD <= 128 ? 4 : 1) void attention_prefill_lds_
     store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
 }
 
+
+// ---------------------------------------------------------------------------------
+// The walk of the kernel above with the blocks brought into LDS by the memory system
+// itself (head sizes 64 and 128, page sizes that are powers of two from 16 up).
+//
+// global_load_lds writes a wave's 64 x 16 bytes to consecutive LDS addresses, whatever
+// global addresses the lanes name: each lane names the 16 bytes that its own operand
+// register will hold, so the block lies in LDS in operand layout without passing through
+// registers, nothing is selected or stored by the waves, and the loads of a block are
+// issued two blocks ahead into a ring of three buffers at no cost in registers.  (Measured
+// on the kernel above: bringing a block in through registers, one block ahead, is a
+// third to two fifths of its time.)
+//
+// For the values to be 16 bytes per lane the keys of a block are assigned to the rows of
+// the two score products so that a lane's eight scores belong to eight consecutive keys:
+// row i of product b is key (i / 4) * 8 + b * 4 + i % 4 of the block.  Lane (r, g) then
+// holds the scores of keys g * 8 .. g * 8 + 7 and needs V^T[d][those keys], one 16-byte
+// run of a page's row.
+//
+// A page that is not there (beyond the context, or given back by a window) is read from
+// page 0 instead: its scores are masked, their weights are exactly zero, and what the
+// cache holds is finite.
+// 64 x 16 bytes from the lanes' global addresses to LDS at `dst` + 16 * lane, without
+// registers in between.  Written as an instruction rather than through the compiler's
+// builtin: the compiler, knowing such a load writes LDS, makes LDS reads wait for every
+// one of them in flight (it cannot always tell the buffers apart), which is the opposite
+// of sending for blocks ahead of time.  The kernel counts these loads itself (s_waitcnt
+// vmcnt) and separates them from the reads by a barrier; "memory" tells the compiler that
+// LDS has changed.
+__device__ __forceinline__ void lds_dma16(const void* src, void* dst) {
+  const unsigned lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)dst;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(src), "s"(lds)
+               : "memory", "m0");
+}
+
+template <int HD>
+__global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attention_prefill_async_kernel(
+    AttentionMfmaArgs args) {
+  constexpr int KS = HD / 32, DB = HD / 16;
+  constexpr int KQ = 2 * KS / 4, VQ = DB / 4;               // slots a wave brings in per block
+  static_assert(HD % 64 == 0, "head sizes in steps of 64");
+  // The ring's three buffers; the loop below is written out three times, each turn with
+  // its buffers named.
+  __shared__ bf16x8 k_lds0[2 * KS][kWave], k_lds1[2 * KS][kWave], k_lds2[2 * KS][kWave];
+  __shared__ bf16x8 v_lds0[DB][kWave], v_lds1[DB][kWave], v_lds2[DB][kWave];
+  const AttentionArgs& a = args.base;
+  const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int r = lane % 16, g = lane / 16;
+  const int group = a.nq / a.nkv;
+  const int heads = a.nkv * args.head_blocks;
+  const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
+  // the first half of the launch takes the long items, longest first, the second half the
+  // short ones, shortest first: a unit's resident workgroups add up to about the same work
+  const int rank = blockIdx.x / heads, front = (args.num_tiles + 1) / 2;
+  const int item = rank < front ? rank : args.num_tiles - 1 - (rank - front);
+  const int kvh = head_slot / args.head_blocks;
+  const int hb = head_slot % args.head_blocks;
+  const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
+            ntok = uniform(args.tiles[item * 3 + 2]);
+  const int* table = a.table + (int64_t)entry * a.table_width;
+  const int P = a.page_size;
+  const int tq = 16 / args.rows_per_token;
+
+  const int ti = wave * tq + r / args.rows_per_token;
+  const int hh = hb * 16 + r % args.rows_per_token;
+  const int head = kvh * group + min(hh, group - 1);
+  const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
+  const int pos_first = uniform(a.positions[tok0]);
+  const int pos_last = pos_first + ntok - 1;
+  const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+  const float scale_log2 = a.scale * 1.44269504088896341f;
+
+  TileState<HD> t;
+  t.pos = row_ok ? pos_first + ti : -1;
+  t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+  const int tile_first = pos_first + wave * tq;
+  const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
+  const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
+  const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+  load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
+                 row_ok, g);
+
+  // Where this lane's 16 bytes of each slot lie, relative to the start of the half of the
+  // block (16 keys) they belong to.  Keys: slot q = b * KS + s0 is product b, elements
+  // g*8*KS + s0*8 .. + 7 of the key in row r.  Values: slot db is head elements
+  // db*16 .. + 15, this lane's row r of them, keys g*8 .. + 7 of the block.
+  const int64_t page_stride = (int64_t)a.nkv * P * HD;         // elements, keys and values alike
+  const bf16_t* k_head = (const bf16_t*)a.k_pages + (int64_t)kvh * P * HD;
+  const bf16_t* v_head = (const bf16_t*)a.v_pages + (int64_t)kvh * HD * P;
+  const bool k_second = r >= 8;          // this lane's keys lie in the block's second 16
+  const bool v_second = g >= 2;
+  unsigned k_off[KQ], v_off[VQ];         // bytes
+#pragma unroll
+  for (int i = 0; i < KQ; ++i) {
+    const int q = wave + 4 * i, b = q / KS, s0 = q % KS;
+    const int key16 = ((r / 4) * 8 + b * 4 + r % 4) % 16;    // inside its half
+    k_off[i] = 2u * (key16 * HD + g * 8 * KS + s0 * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < VQ; ++i)
+    v_off[i] = 2u * (((wave + 4 * i) * 16 + r) * P + (g % 2) * 8);
+
+  const int key_begin = lo_all & ~31;
+  const int nblocks = ((pos_last - key_begin) >> 5) + 1;
+  PageCursor cur{(ConstTable)table, P, pos_last, -1, -1};
+  cur.start(key_begin);
+  // issue the loads of block number `n` (keys key_begin + 32 n ..) into the given buffers;
+  // calls come in order of n, as the cursor needs
+  auto issue = [&](int n, bf16x8 (*kdst)[kWave], bf16x8 (*vdst)[kWave]) {
+    const int kb = key_begin + 32 * n;
+    const int in0 = kb & (P - 1), in1 = (kb + 16) & (P - 1);
+    const int64_t p0 = (int64_t)max(cur.next0, 0) * page_stride, p1 = (int64_t)max(cur.next1, 0) * page_stride;
+    const bf16_t* kb0 = k_head + p0 + in0 * HD;
+    const bf16_t* kb1 = k_head + p1 + in1 * HD;
+    const bf16_t* vb0 = v_head + p0 + in0;
+    const bf16_t* vb1 = v_head + p1 + in1;
+    const char* kbase = (const char*)(k_second ? kb1 : kb0);
+    const char* vbase = (const char*)(v_second ? vb1 : vb0);
+#pragma unroll
+    for (int i = 0; i < KQ; ++i) lds_dma16(kbase + k_off[i], &kdst[wave + 4 * i][0]);
+#pragma unroll
+    for (int i = 0; i < VQ; ++i) lds_dma16(vbase + v_off[i], &vdst[wave + 4 * i][0]);
+    cur.start(kb + 32);
+  };
+  constexpr int kLoads = KQ + VQ;        // vector memory loads a wave has in flight per block
+
+  // One turn: block n is worked on out of (kcur, vcur) while block n + 2 is sent for into
+  // (knext, vnext), the buffers block n - 1 was read from.
+  auto turn = [&](int n, bf16x8 (*kcur)[kWave], bf16x8 (*vcur)[kWave], bf16x8 (*knext)[kWave],
+                  bf16x8 (*vnext)[kWave]) {
+    const int kb = key_begin + 32 * n;
+    if (n + 2 < nblocks) {
+      issue(n + 2, knext, vnext);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoads));      // all but the two youngest blocks
+    } else if (n + 1 < nblocks) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    // Every wave's share of block n is in LDS, and every wave is through with block n - 1.
+    // The bare barrier: __syncthreads would first wait for every load in flight, the two
+    // younger blocks' among them.  The empty statements keep the compiler from moving
+    // LDS reads across it.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kb <= tile_last && kb + 31 >= tile_lo) {
+      KvBlock<HD> b;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = kcur[blk * KS + s0][lane];
+#pragma unroll
+      for (int db = 0; db < DB; ++db) b.v[db] = vcur[db][lane];
+      tile_update<HD, true, true>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
+    }
+  };
+
+  // The query rows are waited for here, once (the empty statement uses them), and not at
+  // their first use inside the loop, where the wait would be for every block in flight
+  // as well; with them gone the vector memory counter counts the blocks' loads alone.
+#pragma unroll
+  for (int s0 = 0; s0 < KS; ++s0) asm volatile("" : "+v"(t.q[s0]));
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  issue(0, k_lds0, v_lds0);
+  if (nblocks > 1) issue(1, k_lds1, v_lds1);
+  for (int n = 0; n < nblocks; n += 3) {
+    turn(n, k_lds0, v_lds0, k_lds2, v_lds2);
+    if (n + 1 < nblocks) turn(n + 1, k_lds1, v_lds1, k_lds0, v_lds0);
+    if (n + 2 < nblocks) turn(n + 2, k_lds2, v_lds2, k_lds1, v_lds1);
+  }
+  const float sum = row_sum<HD>(t);                // by all lanes: it crosses lanes
+  if (row_ok)
+    store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+}
+
 // Query tiles per wavefront: as many as the register file holds accumulators for.
 constexpr int tiles_per_wave(int hd) { return hd <= 32 ? 4 : (hd <= 64 ? 2 : 1); }
 
@@ -317,7 +497,11 @@ template <int HD>
 static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream) {
   if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
   dim3 grid(args.num_tiles * args.base.nkv * args.head_blocks);
-  hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), grid, dim3(256), 0, stream, args);
+  if constexpr (HD % 64 == 0 && HD <= 128) {     // a ring of three blocks fits static LDS
+    hipLaunchKernelGGL((attention_prefill_async_kernel<HD>), grid, dim3(256), 0, stream, args);
+  } else {
+    hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), grid, dim3(256), 0, stream, args);
+  }
   return 0;
 }
 

@@ -25,7 +25,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          # matrix-core results in ordinary vector registers: no copies to and from the
          # accumulation registers around the float32 work between two products
          "-mllvm", "-amdgpu-mfma-vgpr-form",
-         "-Wno-unused-command-line-argument"]
+         "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
 class BuildError(RuntimeError):

@@ -558,7 +558,8 @@ class HipOps:
         # long portions of prompts: a wavefront takes several query tiles and walks alone
         if self._prefill_tiles(batch, a.nkv, group) is not None:
             tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size)
-            tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw)
+            tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw,
+                                                         longest_first=True)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
             m.num_splits = 1
             self._call(self.lib.ts_attention_prefill, byref(m), self._stream())
@@ -593,17 +594,24 @@ class HipOps:
         tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
         return tokens_per_tile if tiles16 * num_kv_heads * -(-group // 16) >= 2048 else None
 
-    def _attention_tiles(self, batch, tokens):
+    def _attention_tiles(self, batch, tokens, longest_first=False):
         """Device list of (entry, first flat token, tokens) cutting every entry of the batch
-        into runs of at most `tokens` consecutive tokens; made once per step and size."""
-        key = ("attn_tiles", tokens)
+        into runs of at most `tokens` consecutive tokens; made once per step and size.
+        `longest_first`: sorted by the number of keys a run's last token sees, most first
+        (the kernels for long portions pair runs from both ends of that order)."""
+        key = ("attn_tiles", tokens, longest_first)
         if key not in batch.plans:
-            tiles = []
+            tiles, keys = [], []
             first = 0
-            for entry, n in enumerate(batch.q_lens):
+            for entry, (n, start) in enumerate(zip(batch.q_lens, batch.starts)):
                 for t0 in range(0, n, tokens):
-                    tiles.append((entry, first + t0, min(tokens, n - t0)))
+                    m = min(tokens, n - t0)
+                    tiles.append((entry, first + t0, m))
+                    keys.append(start + t0 + m)
                 first += n
+            if longest_first:
+                order = sorted(range(len(tiles)), key=lambda i: -keys[i])
+                tiles = [tiles[i] for i in order]
             host = torch.tensor(tiles, dtype=torch.int32)
             batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
         return batch.plans[key]
