@@ -8,6 +8,7 @@
 // TPW tiles; the four waves of a workgroup take neighbouring tiles, so most of their
 // loads meet in the first-level cache.  A tile skips blocks beyond its causal range or
 // before its window, and skips the mask where every key of a block is visible.
+#include <stdlib.h>
 #include "attention_core.h"
 
 template <int HD, int TPW, bool PAGE16>
@@ -344,52 +345,40 @@ __device__ __forceinline__ void lds_dma16(const void* src, void* dst) {
                : "memory", "m0");
 }
 
-template <int HD>
-__global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attention_prefill_async_kernel(
-    AttentionMfmaArgs args) {
+// H = 2: a second set of four waves takes the same four tiles and every second block of
+// their keys (the first set the others), with a ring of its own, and the two partial
+// results of a tile are merged through LDS at the end: twice the waves for a prompt with
+// too few tiles to give every SIMD several.
+//
+// `paired`: a workgroup takes the item at its rank from the front of the sorted list and
+// then the one at the same rank from the back, so every workgroup walks about the same
+// number of blocks wherever it lands.  Unpaired, the first half of the launch takes the
+// long items, longest first, and the second half the short ones, shortest first.
+template <int HD, int H>
+__global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_async_kernel(
+    AttentionMfmaArgs args, int paired) {
   constexpr int KS = HD / 32, DB = HD / 16;
   constexpr int KQ = 2 * KS / 4, VQ = DB / 4;               // slots a wave brings in per block
   static_assert(HD % 64 == 0, "head sizes in steps of 64");
-  // The ring's three buffers; the loop below is written out three times, each turn with
-  // its buffers named.
-  __shared__ bf16x8 k_lds0[2 * KS][kWave], k_lds1[2 * KS][kWave], k_lds2[2 * KS][kWave];
-  __shared__ bf16x8 v_lds0[DB][kWave], v_lds1[DB][kWave], v_lds2[DB][kWave];
+  // a ring buffer: the key slots of a block, then its value slots; three per set of waves
+  constexpr int kSlots = 2 * KS + DB;
+  extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
+  typedef bf16x8 (*Slots)[kWave];
   const AttentionArgs& a = args.base;
-  const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wave_all = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wave = wave_all % 4;             // which of the item's four tiles
+  const int set = H == 1 ? 0 : wave_all / 4; // which of every H key blocks
+  const Slots ring = (Slots)prefill_lds + set * 3 * kSlots;
   const int r = lane % 16, g = lane / 16;
   const int group = a.nq / a.nkv;
   const int heads = a.nkv * args.head_blocks;
   const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
-  // the first half of the launch takes the long items, longest first, the second half the
-  // short ones, shortest first: a unit's resident workgroups add up to about the same work
-  const int rank = blockIdx.x / heads, front = (args.num_tiles + 1) / 2;
-  const int item = rank < front ? rank : args.num_tiles - 1 - (rank - front);
+  const int rank = blockIdx.x / heads;
   const int kvh = head_slot / args.head_blocks;
   const int hb = head_slot % args.head_blocks;
-  const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
-            ntok = uniform(args.tiles[item * 3 + 2]);
-  const int* table = a.table + (int64_t)entry * a.table_width;
   const int P = a.page_size;
   const int tq = 16 / args.rows_per_token;
-
-  const int ti = wave * tq + r / args.rows_per_token;
-  const int hh = hb * 16 + r % args.rows_per_token;
-  const int head = kvh * group + min(hh, group - 1);
-  const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
-  const int pos_first = uniform(a.positions[tok0]);
-  const int pos_last = pos_first + ntok - 1;
-  const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
   const float scale_log2 = a.scale * 1.44269504088896341f;
-
-  TileState<HD> t;
-  t.pos = row_ok ? pos_first + ti : -1;
-  t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
-  const int tile_first = pos_first + wave * tq;
-  const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
-  const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
-  const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
-  load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
-                 row_ok, g);
 
   // Where this lane's 16 bytes of each slot lie, relative to the start of the half of the
   // block (16 keys) they belong to.  Keys: slot q = b * KS + s0 is product b, elements
@@ -410,79 +399,157 @@ __global__ __launch_bounds__(256, HD <= 128 ? 3 : 1) void attention_prefill_asyn
 #pragma unroll
   for (int i = 0; i < VQ; ++i)
     v_off[i] = 2u * (((wave + 4 * i) * 16 + r) * P + (g % 2) * 8);
-
-  const int key_begin = lo_all & ~31;
-  const int nblocks = ((pos_last - key_begin) >> 5) + 1;
-  PageCursor cur{(ConstTable)table, P, pos_last, -1, -1};
-  cur.start(key_begin);
-  // issue the loads of block number `n` (keys key_begin + 32 n ..) into the given buffers;
-  // calls come in order of n, as the cursor needs
-  auto issue = [&](int n, bf16x8 (*kdst)[kWave], bf16x8 (*vdst)[kWave]) {
-    const int kb = key_begin + 32 * n;
-    const int in0 = kb & (P - 1), in1 = (kb + 16) & (P - 1);
-    const int64_t p0 = (int64_t)max(cur.next0, 0) * page_stride, p1 = (int64_t)max(cur.next1, 0) * page_stride;
-    const bf16_t* kb0 = k_head + p0 + in0 * HD;
-    const bf16_t* kb1 = k_head + p1 + in1 * HD;
-    const bf16_t* vb0 = v_head + p0 + in0;
-    const bf16_t* vb1 = v_head + p1 + in1;
-    const char* kbase = (const char*)(k_second ? kb1 : kb0);
-    const char* vbase = (const char*)(v_second ? vb1 : vb0);
-#pragma unroll
-    for (int i = 0; i < KQ; ++i) lds_dma16(kbase + k_off[i], &kdst[wave + 4 * i][0]);
-#pragma unroll
-    for (int i = 0; i < VQ; ++i) lds_dma16(vbase + v_off[i], &vdst[wave + 4 * i][0]);
-    cur.start(kb + 32);
-  };
   constexpr int kLoads = KQ + VQ;        // vector memory loads a wave has in flight per block
 
-  // One turn: block n is worked on out of (kcur, vcur) while block n + 2 is sent for into
-  // (knext, vnext), the buffers block n - 1 was read from.
-  auto turn = [&](int n, bf16x8 (*kcur)[kWave], bf16x8 (*vcur)[kWave], bf16x8 (*knext)[kWave],
-                  bf16x8 (*vnext)[kWave]) {
-    const int kb = key_begin + 32 * n;
-    if (n + 2 < nblocks) {
-      issue(n + 2, knext, vnext);
-      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoads));      // all but the two youngest blocks
-    } else if (n + 1 < nblocks) {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
+  for (int part = 0; part < 2; ++part) {
+    int item;
+    if (paired) {
+      item = part == 0 ? rank : args.num_tiles - 1 - rank;
+      if (part == 1 && item <= rank) break;
     } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
+      if (part == 1) break;
+      const int front = (args.num_tiles + 1) / 2;
+      item = rank < front ? rank : args.num_tiles - 1 - (rank - front);
     }
-    // Every wave's share of block n is in LDS, and every wave is through with block n - 1.
-    // The bare barrier: __syncthreads would first wait for every load in flight, the two
-    // younger blocks' among them.  The empty statements keep the compiler from moving
-    // LDS reads across it.
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    if (kb <= tile_last && kb + 31 >= tile_lo) {
-      KvBlock<HD> b;
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-        for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = kcur[blk * KS + s0][lane];
-#pragma unroll
-      for (int db = 0; db < DB; ++db) b.v[db] = vcur[db][lane];
-      tile_update<HD, true, true>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
-    }
-  };
+    const int entry = uniform(args.tiles[item * 3]), tok0 = uniform(args.tiles[item * 3 + 1]),
+              ntok = uniform(args.tiles[item * 3 + 2]);
+    const int* table = a.table + (int64_t)entry * a.table_width;
 
-  // The query rows are waited for here, once (the empty statement uses them), and not at
-  // their first use inside the loop, where the wait would be for every block in flight
-  // as well; with them gone the vector memory counter counts the blocks' loads alone.
+    const int ti = wave * tq + r / args.rows_per_token;
+    const int hh = hb * 16 + r % args.rows_per_token;
+    const int head = kvh * group + min(hh, group - 1);
+    const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
+    const int pos_first = uniform(a.positions[tok0]);
+    const int pos_last = pos_first + ntok - 1;
+    const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+
+    TileState<HD> t;
+    t.pos = row_ok ? pos_first + ti : -1;
+    t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+    const int tile_first = pos_first + wave * tq;
+    const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
+    const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
+    const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+    load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD,
+                   row_ok, g);
+
+    // The item's blocks of 32 keys, numbered from its first; this set of waves takes
+    // blocks set, set + H, ...: `mine` of them, numbered j here.  Every set makes the same
+    // number of turns (a barrier each), the last of them idle for a set with one block less.
+    const int key_begin = lo_all & ~31;
+    const int nblocks = ((pos_last - key_begin) >> 5) + 1;
+    const int turns = (nblocks + H - 1) / H;
+    const int mine = (nblocks - set + H - 1) / H;
+    const int kb_first = key_begin + 32 * set;
+    PageCursor cur{(ConstTable)table, P, pos_last, -1, -1};
+    cur.start(kb_first);
+    // issue the loads of this set's block j into ring buffer `to`; calls come in order of
+    // j, as the cursor needs
+    auto issue = [&](int j, int to) {
+      const int kb = kb_first + 32 * H * j;
+      const int in0 = kb & (P - 1), in1 = (kb + 16) & (P - 1);
+      const int64_t p0 = (int64_t)max(cur.next0, 0) * page_stride, p1 = (int64_t)max(cur.next1, 0) * page_stride;
+      const bf16_t* kb0 = k_head + p0 + in0 * HD;
+      const bf16_t* kb1 = k_head + p1 + in1 * HD;
+      const bf16_t* vb0 = v_head + p0 + in0;
+      const bf16_t* vb1 = v_head + p1 + in1;
+      const char* kbase = (const char*)(k_second ? kb1 : kb0);
+      const char* vbase = (const char*)(v_second ? vb1 : vb0);
+      const Slots kdst = ring + to * kSlots, vdst = kdst + 2 * KS;
 #pragma unroll
-  for (int s0 = 0; s0 < KS; ++s0) asm volatile("" : "+v"(t.q[s0]));
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  issue(0, k_lds0, v_lds0);
-  if (nblocks > 1) issue(1, k_lds1, v_lds1);
-  for (int n = 0; n < nblocks; n += 3) {
-    turn(n, k_lds0, v_lds0, k_lds2, v_lds2);
-    if (n + 1 < nblocks) turn(n + 1, k_lds1, v_lds1, k_lds0, v_lds0);
-    if (n + 2 < nblocks) turn(n + 2, k_lds2, v_lds2, k_lds1, v_lds1);
+      for (int i = 0; i < KQ; ++i) lds_dma16(kbase + k_off[i], &kdst[wave + 4 * i][0]);
+#pragma unroll
+      for (int i = 0; i < VQ; ++i) lds_dma16(vbase + v_off[i], &vdst[wave + 4 * i][0]);
+      cur.start(kb + 32 * H);
+    };
+
+    // One turn: block j is worked on out of ring buffer `from` while block j + 2 is sent
+    // for into buffer `to`, which block j - 1 was read from.
+    auto turn = [&](int j, int from, int to) {
+      const int kb = kb_first + 32 * H * j;
+      if (j + 2 < mine) {
+        issue(j + 2, to);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoads));    // all but the two youngest blocks
+      } else if (j + 1 < mine) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      // Every wave's share of block j is in LDS, and every wave is through with block
+      // j - 1.  The bare barrier: __syncthreads would first wait for every load in flight,
+      // the two younger blocks' among them.  The empty statements keep the compiler from
+      // moving LDS reads across it.
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (j < mine && kb <= tile_last && kb + 31 >= tile_lo) {
+        const Slots kcur = ring + from * kSlots, vcur = kcur + 2 * KS;
+        KvBlock<HD> b;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int s0 = 0; s0 < KS; ++s0) b.k[blk][s0] = kcur[blk * KS + s0][lane];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) b.v[db] = vcur[db][lane];
+        tile_update<HD, true, true>(t, b, kb, scale_log2, kb + 31 <= tile_first && kb >= tile_lo_last, g);
+      }
+    };
+
+    // The query rows are waited for here, once (the empty statement uses them), and not at
+    // their first use inside the loop, where the wait would be for every block in flight
+    // as well; with them gone the vector memory counter counts the blocks' loads alone.
+#pragma unroll
+    for (int s0 = 0; s0 < KS; ++s0) asm volatile("" : "+v"(t.q[s0]));
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (mine > 0) issue(0, 0);
+    if (mine > 1) issue(1, 1);
+    // written out three times so that every turn's ring buffers are constants
+    for (int j = 0; j < turns; j += 3) {
+      turn(j, 0, 2);
+      if (j + 1 < turns) turn(j + 1, 1, 0);
+      if (j + 2 < turns) turn(j + 2, 2, 1);
+    }
+
+    if constexpr (H == 2) {
+      // The second set hands its partial result over in LDS, in the rings' space: values
+      // [tile][element][lane], then the row statistics.
+      float* lds_o = (float*)prefill_lds;
+      float* lds_ml = lds_o + 4 * DB * 4 * kWave;
+      static_assert(H * 3 * kSlots * kWave * 16 >= (4 * DB * 4 + 4 * 2) * kWave * 4, "merge area");
+      __syncthreads();                             // the rings have been read for the last time
+      if (set == 1) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) lds_o[((wave * DB + db) * 4 + i) * kWave + lane] = t.o[db][i];
+        lds_ml[(wave * 2) * kWave + lane] = t.m;
+        lds_ml[(wave * 2 + 1) * kWave + lane] = t.l;
+      }
+      __syncthreads();
+      if (set == 0) {
+        const float m1 = lds_ml[(wave * 2) * kWave + lane], l1 = lds_ml[(wave * 2 + 1) * kWave + lane];
+        // m is in units of log2; a set that saw no key of this row has m = -inf and weight 0
+        const float m_use = max2(max2(t.m, m1), -1e30f);
+        const float w0 = __builtin_amdgcn_exp2f(t.m - m_use), w1 = __builtin_amdgcn_exp2f(m1 - m_use);
+        t.l = t.l * w0 + l1 * w1;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
+            t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
+          }
+        const float sum = row_sum<HD>(t);          // by all lanes: it crosses lanes
+        if (row_ok)
+          store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+      }
+    } else {
+      const float sum = row_sum<HD>(t);            // by all lanes: it crosses lanes
+      if (row_ok)
+        store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+    }
+    __syncthreads();       // before the next item's blocks are sent for into these buffers
   }
-  const float sum = row_sum<HD>(t);                // by all lanes: it crosses lanes
-  if (row_ok)
-    store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
 }
 
 // Query tiles per wavefront: as many as the register file holds accumulators for.
@@ -493,14 +560,48 @@ extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size) {
   return page_size >= 16 && (page_size & (page_size - 1)) == 0 ? 4 : tiles_per_wave(head_dim);
 }
 
+static int compute_units() {
+  static int cus = 0;       // of the device current when first asked; a host's GPUs are alike
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
+template <int HD, int H>
+static int launch_prefill_async(const AttentionMfmaArgs& args, int paired, hipStream_t stream) {
+  const int heads = args.base.nkv * args.head_blocks;
+  const dim3 grid((paired ? (args.num_tiles + 1) / 2 : args.num_tiles) * heads);
+  const size_t lds = (size_t)H * 3 * (2 * (HD / 32) + HD / 16) * kWave * 16;
+  auto kernel = attention_prefill_async_kernel<HD, H>;
+  static bool raised = false;     // per instantiation
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      TS_FAIL("attention_prefill: cannot raise the LDS limit to %zu bytes", lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(256 * H), lds, stream, args, paired);
+  return 0;
+}
+
 template <int HD>
 static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream) {
   if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
-  dim3 grid(args.num_tiles * args.base.nkv * args.head_blocks);
-  if constexpr (HD % 64 == 0 && HD <= 128) {     // a ring of three blocks fits static LDS
-    hipLaunchKernelGGL((attention_prefill_async_kernel<HD>), grid, dim3(256), 0, stream, args);
+  const int items = args.num_tiles * args.base.nkv * args.head_blocks;
+  if constexpr (HD % 64 == 0 && HD <= 128) {
+    // Few items a compute unit: two sets of waves per item and the items paired, one
+    // workgroup a unit.  Many: one set, three workgroups a unit.
+    int h = items < 6 * compute_units() ? 2 : 1, paired = h == 2;
+    if (const char* e = getenv("TS_PF_MODE")) { h = e[0] - '0'; paired = e[1] - '0'; }
+    return h == 2 ? launch_prefill_async<HD, 2>(args, paired, stream)
+                  : launch_prefill_async<HD, 1>(args, paired, stream);
   } else {
-    hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), grid, dim3(256), 0, stream, args);
+    hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), dim3(items), dim3(256), 0, stream, args);
   }
   return 0;
 }
