@@ -28,6 +28,11 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
+# the vendor library of matrix products, for the plain products with many rows
+LINK = ["-L" + os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib"), "-lhipblaslt",
+        "-Wl,-rpath," + os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")]
+
+
 class BuildError(RuntimeError):
     pass
 
@@ -49,7 +54,7 @@ def source_hash(defines: tuple[str, ...] = ()) -> str:
     for f in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
         h.update(f.name.encode())
         h.update(f.read_bytes())
-    h.update(" ".join(FLAGS + list(defines)).encode())
+    h.update(" ".join(FLAGS + LINK + list(defines)).encode())
     return h.hexdigest()[:16]
 
 
@@ -124,7 +129,7 @@ def build(force: bool = False, verbose: bool = True, jobs: int | None = None) ->
     lib = out_dir / library_name()
     tmp = out_dir / f".{lib.name}.{os.getpid()}"
     _run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", str(tmp)]
-         + [str(o) for o in objs], "linking the kernel library")
+         + [str(o) for o in objs] + LINK, "linking the kernel library")
     os.replace(tmp, lib)
     shutil.rmtree(obj_dir, ignore_errors=True)
     for old in out_dir.glob("libtokensprint_hip.*.so"):

@@ -91,19 +91,38 @@ class HipOps:
             raise KernelError(
                 "the HIP kernels need an AMD GPU (device 'cuda:N'); there is no CPU path")
         self.lib = _load_library()
+        self._device_index = self.device.index if self.device.index is not None \
+            else torch.cuda.current_device()
+        self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
+            lambda index: torch.cuda.current_stream(index).cuda_stream)
         self._attn_chunk = self.lib.ts_attention_mfma_chunk()
+        # for the vendor library's algorithms that want scratch memory during a product
+        self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
 
     # ------------------------------------------------------------ helpers
     def _stream(self):
-        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        # the current stream's handle, by the short way: this runs before every kernel
+        return c_void_p(self._raw_stream(self._device_index))
 
     def _call(self, fn, *args):
         if fn(*args) != 0:
             raise KernelError(self.lib.ts_last_error().decode())
 
     def _check(self, name, t, dtype=None, shape=None, ndim=None):
-        if not isinstance(t, torch.Tensor):
-            raise TypeError(f"{name}: expected a tensor, got {type(t)}")
+        # (written for the case that all is well, which is every call of a working engine:
+        # this runs several times before every kernel)
+        try:
+            ok = t.device == self.device and t.is_contiguous()
+        except AttributeError:
+            raise TypeError(f"{name}: expected a tensor, got {type(t)}") from None
+        if ok and dtype is not None:
+            ok = t.dtype is dtype or (dtype.__class__ is tuple and t.dtype in dtype)
+        if ok and ndim is not None:
+            ok = t.dim() == ndim
+        if ok and shape is not None:
+            ok = t.shape == tuple(shape)
+        if ok:
+            return t
         if t.device != self.device:
             raise ValueError(f"{name}: on {t.device}, kernels run on {self.device}")
         if not t.is_contiguous():
@@ -114,9 +133,7 @@ class HipOps:
                 raise TypeError(f"{name}: dtype {t.dtype}, expected one of {dtypes}")
         if ndim is not None and t.dim() != ndim:
             raise ValueError(f"{name}: {t.dim()} dimensions, expected {ndim}")
-        if shape is not None and tuple(t.shape) != tuple(shape):
-            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
-        return t
+        raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
 
     _FLOATS = (torch.float32, torch.bfloat16)
 
@@ -176,12 +193,15 @@ class HipOps:
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
         if self._library_ok(x, weight):
-            if out_dtype == torch.bfloat16:
-                return torch.matmul(x, weight.t())
-            # the library's float32 sums leave as they are (the output head's logits):
-            # not rounded to bfloat16 and widened, so that logits are of one precision
-            # on both sides of the row count at which the library takes over
-            return torch.mm(x, weight.t(), out_dtype=torch.float32)
+            # the library's float32 sums leave in the type asked for: bfloat16 activations,
+            # float32 logits at the output head (not rounded to bfloat16 and widened, so
+            # that logits are of one precision on both sides of the row count at which
+            # the library takes over)
+            out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+            self._call(self.lib.ts_gemm_library_bf16, _ptr(x), _ptr(weight), _ptr(out),
+                       _TYPE_CODE[out_dtype], M, N, K, _ptr(self._library_workspace),
+                       ctypes.c_size_t(self._library_workspace.numel()), self._stream())
+            return out
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         if self._mfma_ok(x, weight):
             self._call(self.lib.ts_gemm_mfma_bf16, _ptr(x), _ptr(weight), _ptr(out),
