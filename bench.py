@@ -19,7 +19,8 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
 
-def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, model=None):
+def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, model=None,
+                eager=False):
     import torch
     from tokensprint_amd.config import Config
     from tokensprint_amd.engine.assemble import random_model
@@ -33,7 +34,7 @@ def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, m
     config = Config(model=tempfile.gettempdir(), max_model_len=max_len, dtype=model.ctx.dtype,
                     kvcache_block_size=page_size, num_kvcache_blocks=pages,
                     max_num_seqs=max(batch, 1), max_num_batched_tokens=budget,
-                    chunked_prefill=True, eos=-1)
+                    chunked_prefill=True, eos=-1, enforce_eager=eager)
     return model, LLMEngine(model, config)
 
 
@@ -65,6 +66,130 @@ def decode_run(engine, batch, prompt_len, steps, warmup, vocab):
     return dt, (ctx0 + ctx1) / 2.0
 
 
+PRODUCTS = ("linear", "norm_linear", "linear_into_stream", "linear_silu_mul")
+ATTENTION = ("attend", "paged_attention")
+
+
+class Without:
+    """The kernel provider with one kind of call made empty: products, or attention,
+    return a block of zeros of the right shape and launch nothing.  A step captured this
+    way holds the other kernels only, so its replay time is theirs."""
+
+    def __init__(self, ops, kind):
+        import torch
+        self.ops, self.kind, self.torch = ops, kind, torch
+        self.zeros = {}
+
+    def _block(self, shape, dtype):
+        key = (tuple(shape), dtype)
+        if key not in self.zeros:
+            self.zeros[key] = self.torch.zeros(*shape, dtype=dtype, device=self.ops.device)
+        return self.zeros[key]
+
+    def __enter__(self):
+        ops, block = self.ops, self._block
+        if self.kind == "attention":
+            def attend(qkv, batch, table, cache, write_cache, *, num_heads, head_dim, **kw):
+                return block((qkv.shape[0], num_heads, head_dim), qkv.dtype)
+
+            def paged_attention(q, *args, **kw):
+                return block(q.shape, q.dtype)
+            ops.attend, ops.paged_attention = attend, paged_attention
+        else:
+            def linear(x, weight, out_dtype):
+                return block((x.shape[0], weight.shape[0]), out_dtype)
+
+            def linear_silu_mul(x, weight, out_dtype):
+                return block((x.shape[0], weight.shape[0] // 2), out_dtype)
+
+            def norm_linear(resid, delta, norm_weight, eps, weight, out_dtype, silu_mul=False):
+                n = weight.shape[0] // 2 if silu_mul else weight.shape[0]
+                return block((resid.shape[0], n), out_dtype), resid
+
+            ops.linear, ops.linear_silu_mul, ops.norm_linear = linear, linear_silu_mul, norm_linear
+            ops.linear_into_stream = lambda *a, **k: None
+        return self
+
+    def __exit__(self, *exc):
+        for name in (ATTENTION if self.kind == "attention" else PRODUCTS):
+            delattr(self.ops, name)              # the class's method shows again
+
+
+def captured_seconds(runner, batch, reps=20):
+    """Seconds per replay of `runner.run(batch)` captured as a graph."""
+    import torch
+    dev = runner.device
+    side = torch.cuda.Stream(dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        runner.run(batch)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        runner.run(batch)
+    for _ in range(3):
+        graph.replay()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        graph.replay()
+    b.record()
+    torch.cuda.synchronize(dev)
+    return a.elapsed_time(b) * 1e-3 / reps
+
+
+def step_split(model, page, entries_of, max_len):
+    """(seconds of the whole step, of its products, of its attention) for the step that
+    `entries_of(runner)` describes, each from a captured graph: the whole step, the step
+    without attention, the step without products."""
+    from tokensprint_amd.engine.runner import ModelRunner
+    lengths = entries_of(None)
+    pages = sum(-(-n // page) + 1 for n in lengths)
+    runner = ModelRunner(model, page_size=page, num_pages=pages, num_slots=len(lengths))
+    entries = entries_of(runner)
+    width = [-(-max_len // page)] * len(runner.storage.groups)
+    batch = runner.build(entries, width)
+    batch.max_ctx_len = max_len
+    whole = captured_seconds(runner, batch)
+    with Without(model.ctx.ops, "attention"):
+        batch.plans.clear()
+        no_attention = captured_seconds(runner, batch)
+    with Without(model.ctx.ops, "products"):
+        batch.plans.clear()
+        no_products = captured_seconds(runner, batch)
+    batch.plans.clear()
+    return whole, whole - no_products, whole - no_attention
+
+
+def decode_entries(batch, context):
+    """A decode step of `batch` requests that hold `context` tokens each."""
+    from tokensprint_amd.engine.batch import StepEntry
+
+    def make(runner):
+        if runner is None:
+            return [context + 1] * batch
+        out = []
+        for i in range(batch):
+            rc = runner.manager.admit(i)
+            runner.manager.extend(rc, context + 1)
+            out.append(StepEntry(rc, [1], context, [0]))
+        return out
+    return make
+
+
+def prefill_entries(tokens):
+    from tokensprint_amd.engine.batch import StepEntry
+
+    def make(runner):
+        if runner is None:
+            return [tokens]
+        rc = runner.manager.admit(0)
+        runner.manager.extend(rc, tokens)
+        return [StepEntry(rc, [1] * tokens, 0, [tokens - 1])]
+    return make
+
+
 def prefill_run(engine, tokens, vocab, reps=5):
     import torch
     from tokensprint_amd.config import SamplingParams
@@ -82,12 +207,16 @@ def prefill_run(engine, tokens, vocab, reps=5):
     return times[len(times) // 2]
 
 
+def prefill_attention_flops(cfg, T) -> float:
+    """Causal QK^T and PV of one layer for one prompt of T tokens."""
+    return 2 * 2 * cfg["num_attention_heads"] * cfg["head_dim"] * T * (T + 1) / 2
+
+
 def prefill_flops(cfg, layers, T) -> float:
     H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nq, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     per_token = 2 * H * (nq + 2 * nkv) * hd + 2 * nq * hd * H + 3 * 2 * H * I
-    attn = 2 * 2 * nq * hd * T * (T + 1) / 2            # causal QK^T and PV
-    return layers * (per_token * T + attn) + 2 * H * V   # head for the last token only
+    return layers * (per_token * T + prefill_attention_flops(cfg, T)) + 2 * H * V   # head: last token only
 
 
 def main() -> int:
@@ -157,12 +286,30 @@ def main() -> int:
     }
 
     if not args.skip_points:
+        # where the decode step's time goes, from captured steps with one kind of kernel
+        # taken out: products against the weights they stream, attention against the cache
+        context = int(round(mean_tokens / args.batch))
+        whole, t_products, t_attention = step_split(model, page, decode_entries(args.batch, context),
+                                                    ctx_len)
+        out["roofline"]["products_gbs"] = round(wbytes / t_products / 1e9, 1)
+        out["roofline"]["products_us"] = round(t_products * 1e6, 1)
+        out["roofline"]["attention_gbs"] = round(kv_per_token * args.batch * context / t_attention / 1e9, 1)
+        out["roofline"]["attention_us"] = round(t_attention * 1e6, 1)
+        out["roofline"]["step_us_without_host"] = round(whole * 1e6, 1)
+
         T = 2048
         _, pre_engine = make_engine(raw, args.dtype, layers, 1, ctx_len, T, page, model=model)
         sec = prefill_run(pre_engine, T, vocab)
         flops = prefill_flops(raw, layers, T)
+        peak = MFMA_PEAK_TFLOPS[dt_name] * 1e12
         out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
-                          "frac": round(flops / sec / (MFMA_PEAK_TFLOPS[dt_name] * 1e12), 4)}
+                          "frac": round(flops / sec / peak, 4)}
+        attn_flops = layers * prefill_attention_flops(raw, T)
+        _, t_products, t_attention = step_split(model, page, prefill_entries(T), ctx_len)
+        out["prefill"]["products_tflops"] = round((flops - attn_flops) / t_products / 1e12, 1)
+        out["prefill"]["products_us"] = round(t_products * 1e6, 1)
+        out["prefill"]["attention_tflops"] = round(attn_flops / t_attention / 1e12, 1)
+        out["prefill"]["attention_us"] = round(t_attention * 1e6, 1)
         del pre_engine
         points = {}
         for b in (1, 64):       # the same prompts and number of decoded tokens as the headline run
@@ -171,6 +318,14 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * args.steps / d, 1)
             del e
             torch.cuda.empty_cache()
+        # longer contexts: 128 tokens decoded behind prompts that end 256 short of the length
+        for b in (8, 64):
+            for ctx in (2048, 4096):
+                _, e = make_engine(raw, args.dtype, layers, b, ctx_len, 2048, page, model=model)
+                d, _ = decode_run(e, b, ctx - 256, 112, 16, vocab)
+                points[f"decode_b{b}_ctx{ctx}"] = round(b * 112 / d, 1)
+                del e
+                torch.cuda.empty_cache()
         out["points"] = points
     print(json.dumps(out))
     return 0
