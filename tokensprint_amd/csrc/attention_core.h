@@ -136,6 +136,54 @@ __device__ __forceinline__ void load_kv_block(KvBlock<HD>& b, const AttentionArg
   if (PAGE16) cur.start(kb + stride);
 }
 
+// The same block with its keys assigned to the rows of the two score products so that lane
+// (r, g) holds the scores of keys g * 8 .. g * 8 + 7 of the block (row i of product b is
+// key (i / 4) * 8 + b * 4 + i % 4; tile_update's PERM): the lane's share of V^T[d] is then
+// one 16-byte run of a page's row instead of two 8-byte ones, and a block costs a third
+// fewer load instructions, which is what a compute unit's rate of taking them makes a
+// short walk cost.  Page sizes that are powers of two from 16 up; calls in steps of
+// `stride` keys from the cursor's start.
+template <int HD>
+__device__ __forceinline__ void load_kv_block_wide(KvBlock<HD>& b, const AttentionArgs& a,
+                                                   PageCursor& cur, int kvh, int kb, int stride,
+                                                   int r, int g) {
+  constexpr int KS = KvBlock<HD>::KS, DB = KvBlock<HD>::DB;
+  static_assert(HD % 32 == 0, "whole 32-element slices");
+  const bf16_t* kp = (const bf16_t*)a.k_pages;
+  const bf16_t* vp = (const bf16_t*)a.v_pages;
+  const int P = a.page_size;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int page0 = cur.next0, page1 = cur.next1;          // of the block's two 16-key halves
+  const int in0 = kb & (P - 1), in1 = (kb + 16) & (P - 1);
+  // scalar: where the halves' key rows and value columns of this head begin
+  const int64_t h0 = ((int64_t)max(page0, 0) * a.nkv + kvh) * P, h1 = ((int64_t)max(page1, 0) * a.nkv + kvh) * P;
+  const bf16_t* k0 = kp + (h0 + in0) * HD;
+  const bf16_t* k1 = kp + (h1 + in1) * HD;
+  const bf16_t* v0 = vp + h0 * HD + in0;
+  const bf16_t* v1 = vp + h1 * HD + in1;
+  const bool k_second = r >= 8, v_second = g >= 2;         // which half this lane's keys lie in
+  // keys: rows (r / 4) * 8 + r % 4 (product 0) and four further (product 1) of the block,
+  // i.e. row (r % 8 / 4) * 8 + r % 4 [+ 4] of the lane's half
+  const bf16_t* krow = (k_second ? k1 : k0) + (((r % 8) / 4) * 8 + r % 4) * HD + g * 8 * KS;
+  const bf16_t* vcol = (v_second ? v1 : v0) + (int64_t)r * P + (g % 2) * 8;
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) b.k[blk][s] = *(const bf16x8*)(krow + blk * 4 * HD + s * 8);
+#pragma unroll
+  for (int db = 0; db < DB; ++db) b.v[db] = *(const bf16x8*)(vcol + (int64_t)db * 16 * P);
+  if (page0 < 0 || page1 < 0) {      // scalar: only where the context ends or a window has let go
+    const bool k_ok = (k_second ? page1 : page0) >= 0, v_ok = (v_second ? page1 : page0) >= 0;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int s = 0; s < KS; ++s) b.k[blk][s] = k_ok ? b.k[blk][s] : zero8;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) b.v[db] = v_ok ? b.v[db] : zero8;
+  }
+  cur.start(kb + stride);
+}
+
 // One query tile's running state.
 template <int HD>
 struct TileState {

@@ -179,6 +179,12 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   const int key_end = (prep_wave || key_wave) ? 0 : min(c1 * kChunk, last + 1);
   PageCursor cur{(ConstTable)table, a.page_size, last, -1, -1};
   KvBlock<HD> A, B;
+  // head sizes in whole 32-element slices take the blocks with 16-byte value loads
+  constexpr bool kWide = HD % 32 == 0;
+  auto load_block = [&](KvBlock<HD>& b, int kb) {
+    if constexpr (kWide) load_kv_block_wide<HD>(b, a, cur, kvh, kb, stride, r, g);
+    else load_kv_block<HD, true>(b, a, table, cur, kvh, kb, stride, r, g);
+  };
 
   if constexpr (FUSED) {
     // The last wave prepares the query rows for all of them (through LDS): the others
@@ -190,7 +196,7 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     const bool rotate = args.cos != nullptr;
     if (walker) {
       cur.start(key_begin);
-      if (key_begin < key_end) load_kv_block<HD, true>(A, a, table, cur, kvh, key_begin, stride, r, g);
+      if (key_begin < key_end) load_block(A, key_begin);
     }
     if (!walker) {
       prepare_head<HD>(kq, prep_wave ? row_ok : true, prep_weight != nullptr, pw, args.eps, cs, rotate, g);
@@ -246,18 +252,18 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
     }
   } else {
     cur.start(key_begin);
-    if (key_begin < key_end) load_kv_block<HD, true>(A, a, table, cur, kvh, key_begin, stride, r, g);
+    if (key_begin < key_end) load_block(A, key_begin);
     load_query<HD>(t, (const bf16_t*)a.q + ((int64_t)token * a.nq + head) * HD, row_ok, g);
   }
 
   for (int kb = key_begin; kb < key_end; kb += 2 * stride) {
     if (kb + stride < key_end)
-      load_kv_block<HD, true>(B, a, table, cur, kvh, kb + stride, stride, r, g);
-    tile_update<HD>(t, A, kb, scale_log2, kb + 31 <= last && kb >= lo, g);
+      load_block(B, kb + stride);
+    tile_update<HD, false, kWide>(t, A, kb, scale_log2, kb + 31 <= last && kb >= lo, g);
     if (kb + stride >= key_end) break;
     if (kb + 2 * stride < key_end)
-      load_kv_block<HD, true>(A, a, table, cur, kvh, kb + 2 * stride, stride, r, g);
-    tile_update<HD>(t, B, kb + stride, scale_log2, kb + stride + 31 <= last && kb + stride >= lo, g);
+      load_block(A, kb + 2 * stride);
+    tile_update<HD, false, kWide>(t, B, kb + stride, scale_log2, kb + stride + 31 <= last && kb + stride >= lo, g);
   }
   f32x4 (&o)[DB] = t.o;
   float m = t.m, l = row_sum<HD>(t);
