@@ -1,6 +1,6 @@
 """Plain Qwen3 forward: one function per part, whole sequences, no cache, CPU torch.
 
-Every function cites the reference lines (under /root/reference) whose formula it
+Every function cites the lines of the reference's source files whose formula it
 restates.  Inputs are ordinary tensors and numbers; there is no module tree, no
 batching trick and no key/value cache, so a mistake in the engine's cache or batch
 handling cannot be mirrored here.

@@ -8,7 +8,6 @@
 // TPW tiles; the four waves of a workgroup take neighbouring tiles, so most of their
 // loads meet in the first-level cache.  A tile skips blocks beyond its causal range or
 // before its window, and skips the mask where every key of a block is visible.
-#include <stdlib.h>
 #include "attention_core.h"
 
 template <int HD, int TPW, bool PAGE16>
@@ -597,7 +596,6 @@ static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream)
     // Few items a compute unit: two sets of waves per item and the items paired, one
     // workgroup a unit.  Many: one set, three workgroups a unit.
     int h = items < 6 * compute_units() ? 2 : 1, paired = h == 2;
-    if (const char* e = getenv("TS_PF_MODE")) { h = e[0] - '0'; paired = e[1] - '0'; }
     return h == 2 ? launch_prefill_async<HD, 2>(args, paired, stream)
                   : launch_prefill_async<HD, 1>(args, paired, stream);
   } else {
