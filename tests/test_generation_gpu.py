@@ -138,6 +138,36 @@ def test_temperature_sampling_does_not_depend_on_the_batch(setup):
     assert third != together
 
 
+def test_steps_launched_ahead_change_no_token(setup):
+    """Decode steps launched before the host has read the step before them (their tokens
+    taken on the device) against an engine that never does: requests that stop at
+    different lengths or at an end-of-sequence token (whose lane then ran once for
+    nothing), greedy and temperature draws, more requests than may run at once, and a
+    pool so small that requests are preempted."""
+    cfg, d, model, page, prompts, expected = setup
+    L = cfg["max_position_embeddings"]
+    eos = expected[2][5]
+    many = prompts + [p[::-1] for p in prompts]
+    params = [SamplingParams(temperature=0.0 if i % 3 else 0.8, max_tokens=3 + 2 * i,
+                             ignore_eos=i % 4 == 0, seed=i) for i in range(len(many))]
+    for kw in (dict(), dict(max_num_seqs=4), dict(num_kvcache_blocks=-(-64 // page) + 4)):
+        outs, ahead = [], []
+        for on in (False, True):
+            engine = engine_for(model, d, torch.float32, kvcache_block_size=page, max_model_len=L,
+                                eos=eos, seed=5, decode_ahead=on, **kw)
+            outs.append(engine.generate(many, params, use_tqdm=False))
+            ahead.append(engine.num_steps_ahead)
+            engine.runner.manager.check()
+            assert all(p.num_used == 0 for p in engine.runner.manager.pools)
+        assert outs[0] == outs[1], kw
+        assert ahead[0] == 0 and ahead[1] > 0, (kw, ahead)
+    # the first request stops at the end-of-sequence token the plain tokens hold
+    greedy = engine_for(model, d, torch.float32, kvcache_block_size=page, max_model_len=L, eos=eos)
+    out = greedy.generate([prompts[2]] * 3, SamplingParams(temperature=0.0, max_tokens=12),
+                          use_tqdm=False)
+    assert out == [expected[2][:expected[2].index(eos) + 1]] * 3
+
+
 def test_pool_sized_from_free_memory_and_warm_engine(setup):
     """num_kvcache_blocks left at -1: the pool is sized from what a measured largest step
     and the captured graphs leave; every decode bucket is captured before a request."""

@@ -306,6 +306,17 @@ class CacheManager:
         return all(need <= pool.num_free
                    for need, pool in zip(self.pages_needed(rc, new_len), self.pools))
 
+    def can_extend_all(self, wanted: list[tuple[RequestCache, int]]) -> bool:
+        """True if every (request, new length) of `wanted` can be extended, one after the
+        other in any order (pages a window lets go on the way are not counted on)."""
+        need = [0] * len(self.pools)
+        for rc, new_len in wanted:
+            if self._fits_as_is(rc, new_len):
+                continue
+            for g, n in enumerate(self.pages_needed(rc, new_len)):
+                need[g] += max(n, 0)
+        return all(n <= pool.num_free for n, pool in zip(need, self.pools))
+
     def extend(self, rc: RequestCache, new_len: int) -> None:
         """Make positions [rc.num_tokens, new_len) writable; all groups or none."""
         if new_len < rc.num_tokens:

@@ -48,6 +48,7 @@ class Config:
     seed: int = 0
     enable_prefix_caching: bool = False   # share cached full pages between equal prefixes
     warmup: bool = True                   # largest dummy step and graph capture at construction
+    decode_ahead: bool = True             # launch a decode step before the last one's tokens are read
 
     def __post_init__(self) -> None:
         if not os.path.isdir(self.model):

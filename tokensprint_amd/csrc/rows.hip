@@ -23,6 +23,28 @@ extern "C" int ts_embed(const void* table, int table_type, int vocab, const int*
   return 0;
 }
 
+// ---------------------------------------------------------------- tokens drawn on the device
+// ids[i] = drawn[src[i]] where 0 <= src[i] < num_drawn: a step that was launched before
+// the host saw the step before it takes its lanes' tokens from where that step's draw
+// left them.
+__global__ void take_tokens_kernel(int* __restrict__ ids, const int* __restrict__ src,
+                                   const int* __restrict__ drawn, int n, int num_drawn) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int s = src[i];
+  if (s >= 0 && s < num_drawn) ids[i] = drawn[s];
+}
+
+extern "C" int ts_take_tokens(int* ids, const int* src, const int* drawn, int n, int num_drawn,
+                              hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (num_drawn <= 0) TS_FAIL("take_tokens: no drawn tokens to take from");
+  hipLaunchKernelGGL(take_tokens_kernel, dim3((n + 63) / 64), dim3(64), 0, stream, ids, src,
+                     drawn, n, num_drawn);
+  TS_CHECK_LAUNCH("take_tokens");
+  return 0;
+}
+
 // ---------------------------------------------------------------- row gather
 template <typename T>
 __global__ void gather_rows_kernel(const T* __restrict__ x, const int* __restrict__ rows,

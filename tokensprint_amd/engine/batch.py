@@ -58,7 +58,8 @@ def _align(n: int, a: int = 4) -> int:
 def decode_layout(bucket: int, widths: list[int]):
     """Section offsets of a decode-only batch of `bucket` entries, one token each."""
     sizes = [bucket, bucket, bucket, bucket + 1, bucket, bucket, bucket] \
-        + [bucket * w for w in widths] + [bucket, 2 * bucket]     # ... temperatures, keys
+        + [bucket * w for w in widths] + [bucket, 2 * bucket, bucket]   # ... temperatures, keys,
+    #                                                                 lanes to take tokens from
     offs, total = [], 0
     for n in sizes:
         offs.append(total)
@@ -106,11 +107,20 @@ class StaticDecodeBatch:
         self.keys = d[o[8 + G]:o[8 + G] + 2 * B].view(torch.int64)
         self._h_temps = h[o[7 + G]:o[7 + G] + B].view(np.float32)
         self._h_keys = h[o[8 + G]:o[8 + G] + 2 * B].view(np.int64)
+        # lane of the previous step's draw that holds this lane's token; -1: the token
+        # given by the host
+        self.token_sources = d[o[9 + G]:o[9 + G] + B]
+        self._h_sources = h[o[9 + G]:o[9 + G] + B]
+        self._h_sources[:] = -1
 
-    def fill(self, entries, temperatures=None, keys=None) -> None:
+    def fill(self, entries, temperatures=None, keys=None, sources=None) -> None:
+        """`sources[i]`: the lane of the step before whose drawn token is entry i's token
+        (its `tokens[0]` is then a placeholder), or -1."""
         o, B, n = self.offs, self.bucket, len(entries)
         if n > B:
             raise ValueError(f"{n} entries for a static batch of {B} lanes")
+        if sources is not None and len(sources) != n:
+            raise ValueError("one source lane per entry")
         for e in entries:
             for t, w in zip(e.cache.tables, self.widths):
                 if len(t) > w:
@@ -147,6 +157,9 @@ class StaticDecodeBatch:
                     h[base + i * w:base + i * w + max(have, len(t))] = -1
                     h[base + i * w:base + i * w + len(t)] = t
                 self._lane[i][g] = (rc, len(t))
+        self._h_sources[:] = -1
+        if sources is not None:
+            self._h_sources[:n] = sources
         self._h_temps[:] = 0.0
         self._h_keys[:] = 0
         if temperatures is not None:

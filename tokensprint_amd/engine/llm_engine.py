@@ -15,13 +15,28 @@ import torch
 
 from tokensprint_amd.config.engine_config import Config, SamplingParams
 from tokensprint_amd.engine.batch import StepEntry
-from tokensprint_amd.engine.request import Request
+from tokensprint_amd.engine.request import Request, RequestStatus
 from tokensprint_amd.engine.runner import ModelRunner
 from tokensprint_amd.engine.scheduler import Scheduler
 from tokensprint_amd.models.model import Model
 from tokensprint_amd.sampling.sampler import Sampler
 
 log = logging.getLogger(__name__)
+
+
+class _Flight:
+    """A step that has been launched.  `tokens` are its drawn tokens if the host has them
+    already; otherwise they arrive in `host` once `event` has passed."""
+    __slots__ = ("reqs", "sampled_index", "tokens", "host", "event", "positions",
+                 "draw_index", "ahead")
+
+    def __init__(self, reqs, sampled_index, tokens=None, host=None, event=None,
+                 positions=None, draw_index=None, ahead=False):
+        self.reqs, self.sampled_index, self.tokens = reqs, sampled_index, tokens
+        self.host, self.event = host, event
+        self.positions = positions      # per request: position of the token this step computes
+        self.draw_index = draw_index    # per request: index of the completion token it draws
+        self.ahead = ahead              # launched before the step before it was seen
 
 
 class LLMEngine:
@@ -54,6 +69,16 @@ class LLMEngine:
         self.sampler = Sampler(model.ctx.ops, model.ctx.device, config.seed)
         self._next_ordinal = 0
         self.requests: dict[int, Request] = {}
+        # decode steps in flight: the launched step whose tokens have not been read, and
+        # two pinned buffers that take turns receiving a step's tokens
+        self._flight: _Flight | None = None
+        self._landing = []
+        if self.runner.buckets:
+            self._landing = [(torch.empty(self.runner.buckets[-1], dtype=torch.int32,
+                                          pin_memory=True), torch.cuda.Event())
+                             for _ in range(2)]
+        self._turn = 0
+        self.num_steps_ahead = 0        # steps launched before the step before them was seen
 
     @staticmethod
     def largest_step(config: Config) -> tuple[int, int]:
@@ -131,7 +156,7 @@ class LLMEngine:
         return token_ids
 
     def is_finished(self) -> bool:
-        return self.scheduler.is_finished()
+        return self.scheduler.is_finished() and self._flight is None
 
     def add_request(self, prompt: str | list[int], sampling_params: SamplingParams) -> int:
         if isinstance(prompt, str):
@@ -147,7 +172,26 @@ class LLMEngine:
 
     # ------------------------------------------------------------ one step
     def step(self):
-        reqs = self.scheduler.schedule()
+        """Finish one step: the one in flight, or a newly scheduled one.  While a captured
+        decode step runs and the coming step is known without its tokens (nobody can be
+        admitted, the same requests go on decoding), that step is launched first, taking
+        its tokens on the device from the draw before it, so the GPU does not wait for the
+        host's bookkeeping between decode steps."""
+        flight = self._flight or self._launch(self.scheduler.schedule())
+        self._flight = None
+        if flight.event is not None and self.config.decode_ahead:
+            self._flight = self._launch_ahead(flight)
+        return self._finish(flight)
+
+    def _land(self, drawn: torch.Tensor):
+        """Enqueue the copy of a captured step's tokens to the host."""
+        host, event = self._landing[self._turn]
+        self._turn ^= 1
+        host[:drawn.shape[0]].copy_(drawn, non_blocking=True)
+        event.record()
+        return host, event
+
+    def _launch(self, reqs) -> _Flight:
         entries, sampled_index = [], []
         for i, req in enumerate(reqs):
             lo, hi = req.num_cached_tokens, req.num_cached_tokens + req.num_new_tokens
@@ -156,16 +200,73 @@ class LLMEngine:
                 sampled_index.append(i)
             entries.append(StepEntry(req.cache, req.token_ids[lo:hi], lo,
                                      [req.num_new_tokens - 1] if last else []))
-        token_ids = None
         if len(sampled_index) == len(reqs):
             # every entry ends in a draw: a decode step may run, draw included, as one graph
             temps, keys = self.sampler.inputs(reqs)
             drawn = self.runner.decode_and_sample(entries, temps, keys)
             if drawn is not None:
-                token_ids = drawn.tolist()
+                host, event = self._land(drawn)
+                return _Flight(reqs, sampled_index, host=host, event=event,
+                               positions=[e.start for e in entries],
+                               draw_index=[r.num_completion_tokens for r in reqs])
+        logits = self.runner.step(entries)
+        tokens = self.sampler(logits, [reqs[i] for i in sampled_index])
+        return _Flight(reqs, sampled_index, tokens=tokens)
+
+    def _launch_ahead(self, prev: _Flight) -> _Flight | None:
+        """The decode step after `prev`, launched before prev's tokens are known: the
+        requests of prev that go on whatever prev draws, except an end of sequence, whose
+        lane then computes one token that is thrown away.  None if the coming step is the
+        scheduler's to decide (somebody may be admitted, pages run short) or no captured
+        graph serves it."""
+        sch, manager = self.scheduler, self.runner.manager
+        if sch.may_admit():
+            return None
+        reqs, sources, positions, draw_index = [], [], [], []
+        for lane, (req, pos, k) in enumerate(zip(prev.reqs, prev.positions, prev.draw_index)):
+            if req.status is not RequestStatus.RUNNING:
+                continue                 # ended at a step the host has seen since
+            if k + 1 >= req.max_tokens or pos + 2 >= self.config.max_model_len:
+                if sch.waiting:
+                    return None          # its end makes room: the scheduler's step
+                continue                 # ends with the token on its way, whatever it is
+            reqs.append(req)
+            sources.append(lane)
+            positions.append(pos + 1)
+            draw_index.append(k + 1)
+        if not reqs:
+            return None
+        entries = [StepEntry(r.cache, [0], p, [0]) for r, p in zip(reqs, positions)]
+        if not self.runner.fits_captured(entries):
+            return None
+        if not manager.can_extend_all([(r.cache, p + 1) for r, p in zip(reqs, positions)]):
+            return None                  # the scheduler preempts, with everything seen
+        for r, p in zip(reqs, positions):
+            manager.extend(r.cache, p + 1)
+        temps, keys = self.sampler.inputs(reqs, draw_index)
+        drawn = self.runner.decode_and_sample(entries, temps, keys, sources)
+        if drawn is None:
+            raise RuntimeError("a decode step that fitted a captured graph no longer does")
+        host, event = self._land(drawn)
+        self.num_steps_ahead += 1
+        return _Flight(reqs, list(range(len(reqs))), host=host, event=event,
+                       positions=positions, draw_index=draw_index, ahead=True)
+
+    def _finish(self, flight: _Flight):
+        reqs, sampled_index, token_ids = flight.reqs, flight.sampled_index, flight.tokens
         if token_ids is None:
-            logits = self.runner.step(entries)
-            token_ids = self.sampler(logits, [reqs[i] for i in sampled_index])
+            flight.event.synchronize()
+            token_ids = flight.host[:len(reqs)].tolist()
+        if flight.ahead:
+            # a request that ended with the token before this step's: its lane's token is
+            # dropped (its pages went back when it ended; what this step wrote there was
+            # written before anything their next owner runs)
+            keep = [i for i, r in enumerate(reqs) if r.status is RequestStatus.RUNNING]
+            reqs = [reqs[i] for i in keep]
+            token_ids = [token_ids[i] for i in keep]
+            sampled_index = list(range(len(reqs)))
+            for r in reqs:
+                r.num_new_tokens = 1
         self.scheduler.postprocess(reqs, token_ids, sampled_index)
         outputs = [(r.ordinal, r.completion_token_ids) for r in reqs if r.is_finished]
         num_total_tokens = sum(len(r) for r in reqs if r.is_finished)

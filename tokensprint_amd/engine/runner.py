@@ -38,6 +38,7 @@ class ModelRunner:
         self.graph_max_len = graph_max_len
         self.graphs: dict[int, tuple] = {}      # bucket -> (graph, static batch, logits, tokens)
         self._graph_pool = None                 # one memory pool for every captured bucket
+        self._last_drawn = 0                    # entries of the last captured step
         # a part that cannot be captured (it says so) keeps every step eager
         capture = bool(graph_max_len) and self.device.type == "cuda" and model.all_capturable()
         top = min(graph_max_batch, num_slots)
@@ -45,6 +46,10 @@ class ModelRunner:
                                if b <= top}) if capture else []
         self._graph_widths = [-(-graph_max_len // page_size)] * len(self.storage.groups) \
             if capture else []
+        # where every captured step leaves its drawn tokens, lane by lane, and where a
+        # step launched before the host has seen them takes its tokens from
+        self._drawn = torch.zeros(self.buckets[-1], dtype=torch.int32, device=self.device) \
+            if self.buckets else None
 
     @staticmethod
     def pages_that_fit(model: Model, page_size: int, free_bytes: int,
@@ -86,6 +91,10 @@ class ModelRunner:
                 return None
         return next(b for b in self.buckets if b >= len(entries))
 
+    def fits_captured(self, entries) -> bool:
+        """True if `decode_and_sample` would serve these entries from a captured graph."""
+        return self._graph_bucket(entries) is not None
+
     def _capture(self, bucket: int):
         static = StaticDecodeBatch(self.device, bucket, self._graph_widths,
                                    idle_slot=self.storage.idle_slot)
@@ -94,15 +103,20 @@ class ModelRunner:
         torch.cuda.synchronize(self.device)
         side = torch.cuda.Stream(self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
+        ops = self.model.ctx.ops
         with torch.cuda.stream(side):          # loads kernels, fills the batch's launch plans
+            ops.take_tokens(static.batch.token_ids, static.token_sources, self._drawn)
             self.run(static.batch)
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, pool=self._graph_pool):
+            # lanes whose token the step before drew and the host has not seen yet
+            ops.take_tokens(static.batch.token_ids, static.token_sources, self._drawn)
             logits = self.run(static.batch)
             # the draw is part of the captured step: rows with temperature 0 are greedy
-            tokens = self.model.ctx.ops.sample(logits, static.temperatures, static.keys)
+            tokens = ops.sample(logits, static.temperatures, static.keys,
+                                out=self._drawn[:bucket])
         if self._graph_pool is None:
             self._graph_pool = graph.pool()
         self.graphs[bucket] = (graph, static, logits, tokens)
@@ -145,16 +159,23 @@ class ModelRunner:
                 manager.free(e.cache)
         return n * per
 
-    def decode_and_sample(self, entries: list[StepEntry], temperatures, keys):
+    def decode_and_sample(self, entries: list[StepEntry], temperatures, keys, sources=None):
         """One decode step with the draw inside the captured graph: token ids (int32 device
         tensor, one per entry), or None if the step does not fit a captured graph.
-        `temperatures` and `keys` are host sequences, one per entry."""
+        `temperatures` and `keys` are host sequences, one per entry.  The result is a
+        view of the buffer every captured step draws into: read it (or enqueue its copy)
+        before the next captured step.  `sources[i] >= 0` makes entry i's token the one
+        the captured step before this one drew in that lane, so that a step can be
+        launched before the host has seen the last one's tokens."""
         bucket = self._graph_bucket(entries)
         if bucket is None:
             return None
-        return self._replay(bucket, entries, temperatures, keys)[1][:len(entries)]
+        if sources is not None and any(s >= self._last_drawn for s in sources):
+            raise ValueError("a source lane beyond the entries of the step before")
+        return self._replay(bucket, entries, temperatures, keys, sources)[1][:len(entries)]
 
-    def _replay(self, bucket: int, entries: list[StepEntry], temperatures=None, keys=None):
+    def _replay(self, bucket: int, entries: list[StepEntry], temperatures=None, keys=None,
+                sources=None):
         graph, static, logits, tokens = self.graphs.get(bucket) or self._capture(bucket)
         vocab = self.model.spec.vocab_size
         for e in entries:
@@ -163,6 +184,7 @@ class ModelRunner:
             if e.start + 1 > e.cache.num_tokens:
                 raise ValueError(f"request {e.cache.request_id!r}: position {e.start} is not "
                                  "covered by its cache")
-        static.fill(entries, temperatures, keys)
+        static.fill(entries, temperatures, keys, sources)
         graph.replay()
+        self._last_drawn = len(entries)
         return logits[:len(entries)], tokens

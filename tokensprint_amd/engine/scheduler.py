@@ -67,6 +67,11 @@ class Scheduler:
 
     add_sequence = add_request
 
+    def may_admit(self) -> bool:
+        """True if the coming `schedule` could start a waiting request (pages permitting)."""
+        return bool(self.waiting) and len(self.running) < self.max_num_seqs \
+            and self.manager.slots.num_free > 0
+
     # ------------------------------------------------------------ one step
     def schedule(self) -> list[Request]:
         scheduled_running: list[Request] = []

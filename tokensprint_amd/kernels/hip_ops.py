@@ -147,6 +147,14 @@ class HipOps:
                    _ptr(out), T, H, self._stream())
         return out
 
+    def take_tokens(self, token_ids, sources, drawn):
+        """In place: token_ids[i] = drawn[sources[i]] where 0 <= sources[i] < len(drawn)."""
+        self._check("token ids", token_ids, torch.int32, ndim=1)
+        self._check("sources", sources, torch.int32, shape=token_ids.shape)
+        self._check("drawn", drawn, torch.int32, ndim=1)
+        self._call(self.lib.ts_take_tokens, _ptr(token_ids), _ptr(sources), _ptr(drawn),
+                   token_ids.shape[0], drawn.shape[0], self._stream())
+
     def gather_rows(self, x, rows):
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("rows", rows, torch.int32, ndim=1)
@@ -665,14 +673,18 @@ class HipOps:
         return (torch.empty(rows * slices, dtype=torch.float32, device=self.device),
                 torch.empty(rows * slices, dtype=torch.int32, device=self.device))
 
-    def sample(self, logits, temperatures, keys):
+    def sample(self, logits, temperatures, keys, out=None):
         """Row r: greedy if temperatures[r] <= 1e-10, else a draw from
-        softmax(logits[r] / T) with noise keyed by keys[r] (int64 bit pattern)."""
+        softmax(logits[r] / T) with noise keyed by keys[r] (int64 bit pattern).  Into
+        `out` (int32, one per row) if given."""
         self._check("logits", logits, torch.float32, ndim=2)
         R = logits.shape[0]
         self._check("temperatures", temperatures, torch.float32, shape=(R,))
         self._check("keys", keys, torch.int64, shape=(R,))
-        out = torch.empty(R, dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(R, dtype=torch.int32, device=self.device)
+        else:
+            self._check("out", out, torch.int32, shape=(R,))
         part_v, part_i = self._pick_scratch(R, logits.shape[1])
         self._call(self.lib.ts_sample, _ptr(logits), _ptr(temperatures), _ptr(keys), _ptr(out),
                    _ptr(part_v), _ptr(part_i), R, logits.shape[1], self._stream())

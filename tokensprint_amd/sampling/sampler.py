@@ -40,12 +40,15 @@ class Sampler:
     def __init__(self, ops, device, engine_seed: int = 0) -> None:
         self.ops, self.device, self.engine_seed = ops, device, engine_seed
 
-    def inputs(self, requests):
+    def inputs(self, requests, token_indices=None):
         """(temperatures, keys) as host lists, one per request: what the sampling kernel
-        takes.  A greedy request has temperature 0 and needs no key."""
+        takes.  A greedy request has temperature 0 and needs no key.  `token_indices`:
+        which completion token each request draws, if not its next one."""
+        if token_indices is None:
+            token_indices = [r.num_completion_tokens for r in requests]
         temps = [r.temperature if r.temperature > 1e-10 else 0.0 for r in requests]
-        keys = [_signed(noise_key(self.engine_seed, r.seed, r.ordinal, r.num_completion_tokens))
-                if t > 0.0 else 0 for r, t in zip(requests, temps)]
+        keys = [_signed(noise_key(self.engine_seed, r.seed, r.ordinal, k))
+                if t > 0.0 else 0 for r, t, k in zip(requests, temps, token_indices)]
         return temps, keys
 
     def __call__(self, logits: torch.Tensor, requests) -> list[int]:
