@@ -69,6 +69,15 @@ def test_add_rmsnorm_updates_the_residual(ops, gpu_device, dtype):
     torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+def test_take_tokens(ops, gpu_device):
+    ids = torch.arange(100, 109, dtype=torch.int32, device=gpu_device)
+    drawn = torch.tensor([7, 8, 9, 10], dtype=torch.int32, device=gpu_device)
+    src = torch.tensor([-1, 3, 0, -1, 2, 2, 4, -5, 1], dtype=torch.int32, device=gpu_device)
+    ops.take_tokens(ids, src, drawn)
+    # a lane without a source, or with one outside the drawn tokens, keeps its own
+    assert ids.tolist() == [100, 10, 7, 103, 9, 9, 106, 107, 8]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_mul(ops, gpu_device, dtype):
     gu = rand((37, 2 * 150), dtype, gpu_device, 6, scale=3.0)
@@ -135,7 +144,7 @@ def test_linear_bf16_matrix_core_shapes(ops, gpu_device, out_dtype, M, N, K):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 160, 96), (40, 112, 80), (70, 1000, 520),
                                    (40, 3072, 1024), (64, 1000, 2056), (33, 200, 520),
-                                   (5, 304, 3080)])
+                                   (5, 304, 3080), (130, 3072, 1024), (300, 1008, 320)])
 def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
     x = rand((M, K), dtype, gpu_device, 19)
     w = rand((2 * I, K), dtype, gpu_device, 20, scale=0.1)
@@ -149,6 +158,64 @@ def test_linear_silu_mul(ops, gpu_device, dtype, M, I, K):
     else:
         ref = REF.linear_silu_mul(x, w, dtype)
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(300, 400, 320), (70, 1040, 256), (2051, 1024, 2048),
+                                   (513, 4096, 1024), (1000, 48, 4096), (640, 1296, 640)])
+def test_gemm_tiled(ops, gpu_device, out_dtype, M, N, K):
+    """The LDS-tiled product at sizes whose edges cut tiles in both directions and whose
+    tile grids do not divide into the eight regions evenly, with every tile size: against
+    float32 sums of the same bfloat16 operands, and every tile size the same to the bit
+    (one accumulator per element sums K in index order whatever the tile)."""
+    x = rand((M, K), torch.bfloat16, gpu_device, 50)
+    w = rand((N, K), torch.bfloat16, gpu_device, 51, scale=0.05)
+    ref = x.float() @ w.float().T
+    t = dict(rtol=2e-3, atol=2e-3) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    first = None
+    for tile in (0, 1, 2, 3, 4):
+        out = ops.gemm_tiled(x, w, out_dtype, tile=tile)
+        torch.testing.assert_close(out.float(), ref, **t)
+        first = out if first is None else first
+        assert torch.equal(out, first), f"tile {tile} differs"
+    # a row does not depend on the rows beside it
+    one = ops.gemm_tiled(x[M // 3:M // 3 + 1].contiguous(), w, out_dtype)
+    assert torch.equal(one, first[M // 3:M // 3 + 1])
+
+
+@pytest.mark.parametrize("M,I,K", [(130, 112, 256), (2051, 3072, 1024), (300, 1008, 320),
+                                   (65, 16, 256), (700, 2000, 4096)])
+def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
+    """Stacked gate and up weights: the tiles interleave their columns per wave and the
+    epilogue multiplies.  One gate column is made to dominate so that a column paired with
+    the wrong partner, or a tile's columns in the wrong place, shows."""
+    x = rand((M, K), torch.bfloat16, gpu_device, 52)
+    w = rand((2 * I, K), torch.bfloat16, gpu_device, 53, scale=0.05)
+    w[I // 2] *= 8                      # one gate column far above the others
+    w[I + I // 3] *= 8                  # and one up column elsewhere
+    ref = REF.linear_silu_mul(x, w, torch.bfloat16)
+    first = None
+    for tile in (0, 1, 2, 3, 4):
+        out = ops.gemm_tiled(x, w, torch.bfloat16, pair=True, tile=tile)
+        torch.testing.assert_close(out.float(), ref.float(), rtol=2e-2, atol=2e-2)
+        first = out if first is None else first
+        assert torch.equal(out, first), f"tile {tile} differs"
+    # the engine's entry takes this kernel from 65 rows on at weights of this size
+    if 2 * I * K <= ops.TILED_PAIR_WEIGHT:
+        assert torch.equal(ops.linear_silu_mul(x, w, torch.bfloat16), first)
+
+
+def test_gemm_tiled_refuses_what_it_cannot_take(ops, gpu_device):
+    x = rand((100, 200), torch.bfloat16, gpu_device, 54)
+    w = rand((64, 200), torch.bfloat16, gpu_device, 55)
+    with pytest.raises(RuntimeError, match="gemm_tiled"):
+        ops.gemm_tiled(x, w, torch.bfloat16)                  # K not a multiple of 64
+    x = rand((100, 256), torch.bfloat16, gpu_device, 54)
+    w = rand((2 * 24, 256), torch.bfloat16, gpu_device, 55)
+    with pytest.raises(RuntimeError, match="gemm_tiled"):
+        ops.gemm_tiled(x, w, torch.bfloat16, pair=True)       # 24 columns: not a multiple of 16
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ops.gemm_tiled(x, rand((64, 256), torch.bfloat16, gpu_device, 56), torch.float32, pair=True)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
