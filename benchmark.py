@@ -45,6 +45,8 @@ def parse_args(argv=None):
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=-1)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers (random weights only)")
+    ap.add_argument("--decode-ahead", type=_bool, default=True,
+                    help="launch decode steps before the last one's tokens are read")
     return ap.parse_args(argv)
 
 
@@ -89,7 +91,8 @@ def main(args) -> None:
         model=model_dir, enforce_eager=args.enforce_eager, max_model_len=max_model_len,
         max_num_batched_tokens=args.max_num_batched_tokens, max_num_seqs=args.max_num_seqs,
         chunked_prefill=args.chunked_prefill, eos=-1, dtype=model.ctx.dtype,
-        kvcache_block_size=args.page_size, num_kvcache_blocks=args.num_pages))
+        kvcache_block_size=args.page_size, num_kvcache_blocks=args.num_pages,
+        decode_ahead=args.decode_ahead))
     params = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=n) for n in output_lens]
     llm.generate([[1, 2, 3]], SamplingParams(max_tokens=8, ignore_eos=True), use_tqdm=False)
     torch.cuda.synchronize()

@@ -141,6 +141,38 @@ def test_linear_bf16_matrix_core_shapes(ops, gpu_device, out_dtype, M, N, K):
         torch.testing.assert_close(out[M // 2:M // 2 + 1].float(), one.float(), rtol=1e-2, atol=1e-2)
 
 
+def test_library_plan_chosen_by_timing(ops, gpu_device):
+    """A few rows against a large weight with the plan chosen by timing the library's
+    candidates (as the engine does for the decode steps it captures): whichever algorithm
+    wins, the product is the same to rounding, also for later calls with the kept plan
+    and inside a captured graph."""
+    M, N, K = 24, 4096 + 64, 4096         # a shape no other test has planned already
+    x = rand((M, K), torch.bfloat16, gpu_device, 60)
+    w = rand((N, K), torch.bfloat16, gpu_device, 61, scale=0.05)
+    ref = x.float() @ w.float().T
+    ops.timed_plans(True)
+    try:
+        out = ops.linear(x, w, torch.bfloat16)
+    finally:
+        ops.timed_plans(False)
+    torch.testing.assert_close(out.float(), ref, rtol=1e-2, atol=1e-2)
+    again = ops.linear(x, w, torch.bfloat16)
+    assert torch.equal(out, again)
+    side = torch.cuda.Stream(gpu_device)
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream(gpu_device))
+    with torch.cuda.stream(side):
+        ops.linear(x, w, torch.bfloat16)
+    torch.cuda.current_stream(gpu_device).wait_stream(side)
+    with torch.cuda.graph(graph):
+        captured = ops.linear(x, w, torch.bfloat16)
+    for _ in range(3):
+        captured.zero_()
+        graph.replay()
+        torch.cuda.synchronize(gpu_device)
+        assert torch.equal(captured, out)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 160, 96), (40, 112, 80), (70, 1000, 520),
                                    (40, 3072, 1024), (64, 1000, 2056), (33, 200, 520),

@@ -47,8 +47,49 @@ const char* status_name(hipblasStatus_t s) {
     if (s_ != HIPBLAS_STATUS_SUCCESS) TS_FAIL("gemm_library: %s: %s", #call, status_name(s_)); \
   } while (0)
 
+int g_candidates = 1;      // algorithms of the heuristic's list that a plan is chosen from
+
+// Seconds per call of one algorithm on the call's own operands (C is overwritten with the
+// same product every time), or a negative number if the library refuses it.  Before every
+// timed call `flush` is overwritten: a decode step reads each weight once, from HBM, and a
+// weight left in the memory-side cache by the call before would favour other algorithms
+// than the ones that are fastest then.
+double time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulAlgo_t& algo,
+                 const void* a, const void* w, void* c, void* workspace, size_t workspace_bytes,
+                 void* flush, size_t flush_bytes, hipStream_t stream) {
+  const float alpha = 1.f, beta = 0.f;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return -1.;
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return -1.; }
+  double best = -1.;
+  for (int i = 0; i < 4; ++i) {         // the first call is a warm-up (code, descriptors)
+    bool ok = flush == nullptr || hipMemsetAsync(flush, i, flush_bytes, stream) == hipSuccess;
+    ok = ok && hipEventRecord(e0, stream) == hipSuccess;
+    ok = ok && hipblasLtMatmul(handle, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &algo,
+                               workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+    float ms = 0.f;
+    ok = ok && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    if (!ok) { best = -1.; break; }
+    if (i > 0 && (best < 0. || ms * 1e-3 < best)) best = ms * 1e-3;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return best;
+}
+
+// The plan of one (rows, columns, inner size, output type).  The heuristic's first choice
+// is right for the shapes of prompts; for a few rows against a large weight (decode steps
+// of 9 to 64 requests at the 8B and 32B shapes) it has been seen at a third of the rate of
+// the list's best, so where the caller has asked for it (ts_gemm_library_candidates: the
+// engine does while it prepares the decode steps it captures, whose plans are used for
+// the rest of the run) the first entries of the list are run on the call's own operands
+// and the fastest is kept.  Timing costs some ten milliseconds a plan, too much for a shape
+// that a step meets once.  Under stream capture nothing can be timed and the first
+// choice stands.
 int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int c_type,
-              size_t workspace_bytes) {
+              size_t workspace_bytes, const void* a, const void* w, void* c, void* workspace,
+              hipStream_t stream) {
   const hipDataType out = c_type == TS_BF16 ? HIP_R_16BF : HIP_R_32F;
   TS_BLAS(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   const hipblasOperation_t t = HIPBLAS_OP_T, n = HIPBLAS_OP_N;
@@ -61,20 +102,55 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int c_type
   TS_BLAS(hipblasLtMatmulPreferenceCreate(&pref));
   TS_BLAS(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
                                                 &workspace_bytes, sizeof(workspace_bytes)));
-  hipblasLtMatmulHeuristicResult_t found;
+  constexpr int kMost = 16;
+  hipblasLtMatmulHeuristicResult_t found[kMost];
   int count = 0;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  const bool few_rows = M <= 64 && (int64_t)N * K >= (1 << 23);
+  const bool tune = few_rows && g_candidates > 1 &&
+                    hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+                    capturing == hipStreamCaptureStatusNone;
+  const int ask = tune ? (g_candidates < kMost ? g_candidates : kMost) : 1;
   const hipblasStatus_t s = hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.w, p.a, p.c, p.c,
-                                                            pref, 1, &found, &count);
+                                                            pref, ask, found, &count);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (s != HIPBLAS_STATUS_SUCCESS || count < 1)
     TS_FAIL("gemm_library: the library has no algorithm for M=%d N=%d K=%d (%s)", M, N, K,
             status_name(s));
-  p.algo = found.algo;
-  p.workspace = found.workspaceSize;
+  int best = 0;
+  if (tune && count > 1) {
+    // larger than the memory-side cache; given back before this returns
+    const size_t flush_bytes = (size_t)512 << 20;
+    void* flush = nullptr;
+    if (hipMalloc(&flush, flush_bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      flush = nullptr;
+    }
+    // the first choice stands unless another is ahead by more than the timing's noise
+    double best_seconds = -1.;
+    for (int i = 0; i < count; ++i) {
+      if (found[i].workspaceSize > workspace_bytes) continue;
+      const double sec = time_algo(handle, p, found[i].algo, a, w, c, workspace, workspace_bytes,
+                                   flush, flush_bytes, stream);
+      if (sec <= 0.) continue;
+      if (best_seconds < 0. || sec < 0.95 * best_seconds) { best_seconds = sec; best = i; }
+    }
+    if (flush != nullptr) {
+      (void)hipStreamSynchronize(stream);
+      (void)hipFree(flush);
+    }
+  }
+  p.algo = found[best].algo;
+  p.workspace = found[best].workspaceSize;
   return 0;
 }
 
 }  // namespace
+
+// How many entries of the heuristic's list a plan for few rows is chosen from by timing
+// them, from now on (1, the default: the first is taken untimed).  Plans already made keep
+// their choice.
+extern "C" void ts_gemm_library_candidates(int n) { g_candidates = n < 1 ? 1 : n; }
 
 // `workspace`: device memory of `workspace_bytes` for the library's use during the call,
 // the same for every call on a stream (calls on one stream run one after the other).
@@ -101,7 +177,7 @@ extern "C" int ts_gemm_library_bf16(const void* a, const void* w, void* c, int c
     auto it = g_plans[device].find(key);
     if (it == g_plans[device].end()) {
       Plan p;
-      if (make_plan(handle, p, M, N, K, c_type, workspace_bytes)) return -1;
+      if (make_plan(handle, p, M, N, K, c_type, workspace_bytes, a, w, c, workspace, stream)) return -1;
       it = g_plans[device].emplace(key, p).first;
     }
     plan = &it->second;     // entries of an unordered_map stay where they are

@@ -220,6 +220,13 @@ class HipOps:
                        self._stream())
         return out
 
+    def timed_plans(self, on: bool) -> None:
+        """While on, the library products of few rows that are met for the first time have
+        their algorithm chosen by timing the first entries of the library's list instead
+        of taking the first (some ten milliseconds a shape: for shapes that will be used
+        for the rest of the run, i.e. the decode steps that are captured)."""
+        self.lib.ts_gemm_library_candidates(8 if on else 1)
+
     def gemm_tiled(self, x, weight, out_dtype, pair=False, tile=0):
         """The LDS-tiled product for many rows: x [M, K] bfloat16, weight [N, K] bfloat16
         (with `pair` [2 N, K], gate rows then up rows, and the result is silu(gate) * up).
