@@ -79,12 +79,13 @@ double time_algo(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulA
 }
 
 // The plan of one (rows, columns, inner size, output type).  The heuristic's first choice
-// is right for the shapes of prompts; for a few rows against a large weight (decode steps
-// of 9 to 64 requests at the 8B and 32B shapes) it has been seen at a third of the rate of
-// the list's best, so where the caller has asked for it (ts_gemm_library_candidates: the
-// engine does while it prepares the decode steps it captures, whose plans are used for
-// the rest of the run) the first entries of the list are run on the call's own operands
-// and the fastest is kept.  Timing costs some ten milliseconds a plan, too much for a shape
+// is mostly right, but for a few rows against a large weight (decode steps of 9 to 64
+// requests at the 8B and 32B shapes) it has been seen at a third of the rate of the list's
+// best, and for 8,192 rows at N = 5,120 at three quarters.  So where the caller has asked
+// for it (ts_gemm_library_candidates: the engine does during its warm-up, whose largest
+// step and captured decode steps have the shapes the run is made of) the first entries of
+// the list are run on the call's own operands and the fastest is kept, for weights from
+// 2^20 elements.  Timing costs ten to a hundred milliseconds a plan, too much for a shape
 // that a step meets once.  Under stream capture nothing can be timed and the first
 // choice stands.
 int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int c_type,
@@ -106,8 +107,7 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int c_type
   hipblasLtMatmulHeuristicResult_t found[kMost];
   int count = 0;
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  const bool few_rows = M <= 64 && (int64_t)N * K >= (1 << 23);
-  const bool tune = few_rows && g_candidates > 1 &&
+  const bool tune = g_candidates > 1 && (int64_t)N * K >= (1 << 20) &&
                     hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
                     capturing == hipStreamCaptureStatusNone;
   const int ask = tune ? (g_candidates < kMost ? g_candidates : kMost) : 1;

@@ -47,6 +47,16 @@ class LLMEngine:
         page = config.kvcache_block_size
         on_gpu = model.ctx.device.type == "cuda"
         graph_len = None if config.enforce_eager or not on_gpu else config.max_model_len
+        # the shapes that the warm-up meets (the largest step, the captured decode steps)
+        # are the ones the run is made of: their library plans are worth timing
+        timed_plans = getattr(model.ctx.ops, "timed_plans", lambda on: False)
+        before = timed_plans(config.warmup and on_gpu)
+        try:
+            self._set_up(model, config, page, on_gpu, graph_len)
+        finally:
+            timed_plans(before)
+
+    def _set_up(self, model, config, page, on_gpu, graph_len) -> None:
         num_pages = config.num_kvcache_blocks
         if num_pages < 0:
             num_pages = self._pages_from_free_memory(model, config, graph_len)

@@ -104,14 +104,14 @@ class ModelRunner:
         side = torch.cuda.Stream(self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         ops = self.model.ctx.ops
-        timed_plans = getattr(ops, "timed_plans", lambda on: None)
-        timed_plans(True)                      # this step's shapes stay for the rest of the run
+        timed_plans = getattr(ops, "timed_plans", lambda on: False)
+        before = timed_plans(True)             # this step's shapes stay for the rest of the run
         try:
             with torch.cuda.stream(side):      # loads kernels, fills the batch's launch plans
                 ops.take_tokens(static.batch.token_ids, static.token_sources, self._drawn)
                 self.run(static.batch)
         finally:
-            timed_plans(False)
+            timed_plans(before)
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()

@@ -98,6 +98,7 @@ class HipOps:
         self._attn_chunk = self.lib.ts_attention_mfma_chunk()
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
+        self._timed_plans = False
 
     # ------------------------------------------------------------ helpers
     def _stream(self):
@@ -220,12 +221,16 @@ class HipOps:
                        self._stream())
         return out
 
-    def timed_plans(self, on: bool) -> None:
-        """While on, the library products of few rows that are met for the first time have
-        their algorithm chosen by timing the first entries of the library's list instead
-        of taking the first (some ten milliseconds a shape: for shapes that will be used
-        for the rest of the run, i.e. the decode steps that are captured)."""
+    def timed_plans(self, on: bool) -> bool:
+        """While on, the library products that are met for the first time have their
+        algorithm chosen by timing the first entries of the library's list instead of
+        taking the first (ten to a hundred milliseconds a shape: for shapes that will be
+        used for the rest of the run, i.e. the warm-up's largest step and the decode
+        steps that are captured).  Returns what it was before."""
+        before = self._timed_plans
+        self._timed_plans = bool(on)
         self.lib.ts_gemm_library_candidates(8 if on else 1)
+        return before
 
     def gemm_tiled(self, x, weight, out_dtype, pair=False, tile=0):
         """The LDS-tiled product for many rows: x [M, K] bfloat16, weight [N, K] bfloat16
