@@ -102,9 +102,35 @@ __global__ void qk_prepare_kernel(QkPrepareArgs a) {
 // The same for bfloat16 activations and head sizes 16, 32, 64, 128, 256: hd/8 lanes per
 // head, eight consecutive elements per lane in one 16-byte load, the rotation partner
 // (the element hd/2 further) fetched from the lane hd/16 further.  `with_v` = 0 leaves the
-// value heads to v_store_tile_kernel.
+// value heads to the workgroups that store them tile by tile (v_store_tile).
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_qk;
 typedef __attribute__((ext_vector_type(4))) float f32x4_qk;
+
+// Values of many tokens into their pages (bfloat16 to bfloat16).  A page holds values
+// transposed, [head element][position], so a token's head vector lands two bytes at a
+// time, hd rows apart: here 16 lanes take 16 consecutive tokens for the same 8 head
+// elements, and since consecutive tokens of a prompt sit at consecutive positions, the 16
+// two-byte stores of one row fall into one 32-byte run of the page.  A workgroup of 256
+// takes (tile of 16 tokens, key/value head); its 16 lane groups take 8 head elements
+// each, in rounds.
+__device__ __forceinline__ void v_store_tile(const QkPrepareArgs& a, int tile, int kvh) {
+  const int j = threadIdx.x % 16;
+  const int t = tile * 16 + j;
+  if (t >= a.num_tokens) return;
+  const int pos = a.positions[t];
+  const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
+  if (page < 0) return;
+  const int hd = a.hd;
+  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * (a.nq + 2 * a.nkv) * hd +
+                      (int64_t)(a.nq + a.nkv + kvh) * hd;
+  bf16_t* dst = (bf16_t*)a.v_dst + ((int64_t)page * a.nkv + kvh) * a.page_size * hd +
+                pos % a.page_size;
+  for (int d0 = (threadIdx.x / 16) * 8; d0 < hd; d0 += 128) {
+    const bf16x8_qk x = *(const bf16x8_qk*)(src + d0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[(int64_t)(d0 + i) * a.page_size] = x[i];
+  }
+}
 
 // A thread goes through its piece (N of them: one was measured best, more waves do
 // better than longer ones) in three rounds: everything that hangs on nothing (the
@@ -113,7 +139,14 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_qk;
 // trips to memory, not one per use.
 template <typename TC, int N>
 __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, int lanes_log2,
-                                                             int with_v) {
+                                                             int with_v, int v_first_block) {
+  // with_v = 0 and v_first_block >= 0: the workgroups from that one on store the values
+  // tile by tile (one launch for both: a second launch costs more than its work here)
+  if (v_first_block >= 0 && (int)blockIdx.x >= v_first_block) {
+    const int idx = blockIdx.x - v_first_block;
+    v_store_tile(a, idx / a.nkv, idx % a.nkv);
+    return;
+  }
   const int L = 1 << lanes_log2;                     // lanes per head
   const int heads_per_wave = kWave >> lanes_log2;
   const int lane = threadIdx.x % kWave;
@@ -226,32 +259,6 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(QkPrepareArgs a, in
   }
 }
 
-// Values of many tokens into their pages (bfloat16 to bfloat16).  A page holds values
-// transposed, [head element][position], so a token's head vector lands two bytes at a
-// time, hd rows apart: here 16 lanes take 16 consecutive tokens for the same 8 head
-// elements, and since consecutive tokens of a prompt sit at consecutive positions, the 16
-// two-byte stores of one row fall into one 32-byte run of the page.  Workgroup (tile of
-// 16 tokens, key/value head); its 16 lane groups take 8 head elements each, in rounds.
-__global__ __launch_bounds__(256) void v_store_tile_kernel(QkPrepareArgs a) {
-  const int j = threadIdx.x % 16;
-  const int t = blockIdx.x * 16 + j;
-  const int kvh = blockIdx.y;
-  if (t >= a.num_tokens) return;
-  const int pos = a.positions[t];
-  const int page = a.table[(int64_t)a.entry_of_token[t] * a.table_width + pos / a.page_size];
-  if (page < 0) return;
-  const int hd = a.hd;
-  const bf16_t* src = (const bf16_t*)a.qkv + (int64_t)t * (a.nq + 2 * a.nkv) * hd +
-                      (int64_t)(a.nq + a.nkv + kvh) * hd;
-  bf16_t* dst = (bf16_t*)a.v_dst + ((int64_t)page * a.nkv + kvh) * a.page_size * hd +
-                pos % a.page_size;
-  for (int d0 = (threadIdx.x / 16) * 8; d0 < hd; d0 += 128) {
-    const bf16x8_qk x = *(const bf16x8_qk*)(src + d0);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) dst[(int64_t)(d0 + i) * a.page_size] = x[i];
-  }
-}
-
 extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_type,
                              hipStream_t stream) {
   QkPrepareArgs a = *args;
@@ -268,22 +275,19 @@ extern "C" int ts_qk_prepare(const QkPrepareArgs* args, int act_type, int cache_
   const int waves_per_block = 4;
   if (act_type == TS_BF16 && a.hd >= 16 && a.hd <= 256 && (a.hd & (a.hd - 1)) == 0 &&
       ((uintptr_t)a.qkv & 15) == 0 && ((uintptr_t)a.q_out & 15) == 0) {
-    // portions of prompts: the values go tile by tile (a second launch pays from a few
-    // tiles on)
-    const bool v_tiles = a.store_kv && a.paged && cache_type == TS_BF16 && a.num_tokens >= 64 &&
-                         a.nkv <= 65535;
+    // portions of prompts: the values go tile by tile, by further workgroups of the same
+    // launch
+    const bool v_tiles = a.store_kv && a.paged && cache_type == TS_BF16 && a.num_tokens >= 64;
     const int lanes_log2 = __builtin_ctz(a.hd / 8);
     const int heads_per_block = waves_per_block * (kWave >> lanes_log2);
     const int64_t vec_items = v_tiles ? (int64_t)a.num_tokens * (a.nq + a.nkv) : items;
     const int64_t vblocks = (vec_items + heads_per_block - 1) / heads_per_block;
-    if (vblocks > 2147483647LL) TS_FAIL("qk_prepare: too many tokens");
+    const int64_t tiles = v_tiles ? (int64_t)((a.num_tokens + 15) / 16) * a.nkv : 0;
+    if (vblocks + tiles > 2147483647LL) TS_FAIL("qk_prepare: too many tokens");
     TS_DISPATCH_TYPE(cache_type, TC,
-        hipLaunchKernelGGL((qk_prepare_vec_kernel<TC, 1>), dim3((unsigned)vblocks),
+        hipLaunchKernelGGL((qk_prepare_vec_kernel<TC, 1>), dim3((unsigned)(vblocks + tiles)),
                            dim3(waves_per_block * kWave), 0, stream, a, lanes_log2,
-                           v_tiles ? 0 : 1));
-    if (v_tiles)
-      hipLaunchKernelGGL(v_store_tile_kernel, dim3((a.num_tokens + 15) / 16, a.nkv), dim3(256),
-                         0, stream, a);
+                           v_tiles ? 0 : 1, v_tiles ? (int)vblocks : -1));
     TS_CHECK_LAUNCH("qk_prepare");
     return 0;
   }
