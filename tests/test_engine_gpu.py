@@ -182,10 +182,10 @@ def test_eps_of_the_per_head_norms_shows(name, dtype, tmp_path, gpu_device):
     drives.compare(col, ref, rtol, atol)
 
 
-@pytest.fixture(scope="module")
-def wide_bfloat16(tmp_path_factory, gpu_device):
-    cfg, seed, page = GPU_ONLY["F"]
-    d = tmp_path_factory.mktemp("wideF")
+@pytest.fixture(scope="module", params=["E", "F"])
+def wide_bfloat16(request, tmp_path_factory, gpu_device):
+    cfg, seed, page = GPU_ONLY[request.param]
+    d = tmp_path_factory.mktemp("wide" + request.param)
     write_random_model(d, cfg, seed, torch.bfloat16)
     pcfg, w = plain.read_model_dir(d)
     _, model = load_model(d, torch.bfloat16, gpu_device)
@@ -194,11 +194,13 @@ def wide_bfloat16(tmp_path_factory, gpu_device):
 
 
 @pytest.mark.parametrize("captured", [False, True], ids=["eager", "captured"])
-@pytest.mark.parametrize("lanes", [4, 5, 8, 9, 16, 17, 64, 65])
+@pytest.mark.parametrize("lanes", [4, 5, 8, 9, 16, 17, 32, 33, 64, 65])
 def test_decode_lanes_on_both_sides_of_each_kernel_choice(wide_bfloat16, lanes, captured):
     """Which kernel serves a product depends on the number of rows: the output head goes
     to the library from 5 rows, the layer products of this width from 9, those with a
-    short K from 17, everything from 65.  A decode step with one lane fewer and one lane
+    short K from 17, everything from 65 (the 8B width, F); at the 0.6B width (E) the layer
+    products are this engine's up to 64 rows, with more tiles of rows per workgroup from 17
+    and from 33.  A decode step with one lane fewer and one lane
     more than each of these must give the plain logits, eagerly and from a captured graph."""
     from tokensprint_amd.engine import StepEntry
     model, page, tokens, ref = wide_bfloat16
