@@ -593,11 +593,16 @@ static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream)
   if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
   const int items = args.num_tiles * args.base.nkv * args.head_blocks;
   if constexpr (HD % 64 == 0 && HD <= 128) {
-    // Few items a compute unit: two sets of waves per item and the items paired, one
-    // workgroup a unit.  Many: one set, three workgroups a unit.
-    int h = items < 6 * compute_units() ? 2 : 1, paired = h == 2;
-    return h == 2 ? launch_prefill_async<HD, 2>(args, paired, stream)
-                  : launch_prefill_async<HD, 1>(args, paired, stream);
+    // Up to two items a compute unit: two sets of waves per item, and the items paired (a
+    // long one and a short one per workgroup) once there are more items than units, so
+    // that one round of workgroups of equal length fills the chip.  More: one set, three
+    // workgroups a unit, longest first.  (Measured at 16 query and 8 key/value heads of
+    // 128: 1,024 tokens 21.5 us with two sets unpaired, 25.3 paired; 1,536 tokens 34.0
+    // paired, 35.7 unpaired; 2,048 tokens 42.6 paired, 48.8 with one set; 2,560 tokens 63.9
+    // with one set, 92.7 with two sets paired, which then need a second round.)
+    const int units = compute_units();
+    if (items <= 2 * units) return launch_prefill_async<HD, 2>(args, items > units, stream);
+    return launch_prefill_async<HD, 1>(args, 0, stream);
   } else {
     hipLaunchKernelGGL((attention_prefill_lds_kernel<HD>), dim3(items), dim3(256), 0, stream, args);
   }

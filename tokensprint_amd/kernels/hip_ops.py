@@ -663,11 +663,17 @@ class HipOps:
         self._call(self.lib.ts_attention_mfma, byref(m), self._stream())
 
     def _prefill_tiles(self, batch, num_kv_heads, group):
-        """Tokens per 16-row tile if the step is one of long portions of prompts (enough
-        tiles to fill the chip with wavefronts that walk alone), else None."""
+        """Tokens per 16-row tile if the step holds portions of prompts (enough 16-row
+        tiles for the kernel whose waves share key/value blocks through LDS), else None.
+        Measured at 16 query and 8 key/value heads of 128 against the general kernel: one
+        portion of 256 tokens 11.0 against 16.6 us, 1,024 tokens 21.5 against 34.4, 1,536
+        tokens 34.0 against 96.8; below that the two are equal."""
         tokens_per_tile = 16 // min(group, 16)
         tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
-        return tokens_per_tile if tiles16 * num_kv_heads * -(-group // 16) >= 2048 else None
+        waves = tiles16 * num_kv_heads * -(-group // 16)
+        # a step of single tokens only takes it where the chip is full without splitting keys
+        enough = 256 if batch.max_q_len >= 32 else 2048
+        return tokens_per_tile if waves >= enough else None
 
     def _attention_tiles(self, batch, tokens, longest_first=False):
         """Device list of (entry, first flat token, tokens) cutting every entry of the batch
