@@ -105,7 +105,8 @@ class TorchOps:
         return q
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
-               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window):
+               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
+               defer_merge=False):
         q = self.qk_norm_rope_store(
             qkv, batch, table, cache if write_cache else None, num_heads=num_heads,
             num_kv_heads=kv_in_row, head_dim=head_dim, q_weight=q_weight, k_weight=k_weight,

@@ -612,6 +612,72 @@ def test_attend_decode_long_contexts_split_and_merge(ops, gpu_device, window, fu
     torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("window", [None, 1000])
+@pytest.mark.parametrize("nq,nkv,hd,hidden,spans", [
+    (16, 8, 128, 1024, [(5000, 1), (2047, 1), (3, 1), (2049, 1)]),
+    (16, 8, 128, 1024, [(777, 1)]),
+    (32, 8, 128, 4096, [(3000, 1), (129, 1), (4100, 1), (0, 1), (640, 1), (2500, 1), (77, 1),
+                        (1024, 1)]),
+    (16, 8, 128, 1024, [(3000, 1), (129, 1), (4100, 1), (0, 1), (640, 1), (2500, 1), (77, 1),
+                        (1024, 1), (900, 1), (31, 1), (4000, 1)]),
+    (40, 2, 64, 520, [(1500, 1), (300, 1)]),
+])
+def test_output_projection_merges_the_key_splits_itself(ops, gpu_device, monkeypatch, nq, nkv, hd,
+                                                        hidden, spans, window):
+    """A decode step whose keys are split over workgroups: with the merge deferred, the
+    output projection in its tail form merges the partial results as it loads its rows.
+    Stream, prepared rows and sums of squares must be, bit for bit, what the merge kernel
+    followed by the tail form leaves; and a deferred merge that another call meets (a
+    plain product here) is run before that call."""
+    from tokensprint_amd.kernels.stream import NormHint
+    dtype, page = torch.bfloat16, 16
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=81)
+    T = batch.num_tokens
+    group = nq // nkv
+    assert ops._decode_splits(T * nkv * -(-group // 16), batch.max_ctx_len) > 1
+    qkv = rand((T, (nq + 2 * nkv) * hd), dtype, gpu_device, 82)
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 83)
+    angles = torch.outer(torch.arange(5100, dtype=torch.float32),
+                         1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    kw = dict(num_heads=nq, num_kv_heads=nkv, kv_in_row=nkv, head_dim=hd, q_weight=wq,
+              k_weight=wq, eps=1e-6, cos_sin=cos_sin, scale=hd ** -0.5, window=window)
+    w_o = rand((hidden, nq * hd), dtype, gpu_device, 84, scale=0.05)
+    norm_w = 1 + 0.1 * rand((hidden,), torch.float32, gpu_device, 85)
+    w_next = rand((2 * 96, hidden), dtype, gpu_device, 86, scale=0.05)
+    hint = NormHint(norm_w, 1e-6, w_next, True)
+    resid0 = rand((T, hidden), torch.float32, gpu_device, 87)
+
+    # (the provider defers only up to the few rows for which it pays; here every size)
+    monkeypatch.setattr(ops, "merged_rows", 16)
+
+    def run(defer):
+        mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                           cache.k_pages.clone(), cache.v_pages.clone())
+        o = ops.attend(qkv, batch, table, mine, True, defer_merge=defer, **kw).view(T, nq * hd)
+        assert (ops._unmerged is not None) == defer
+        resid = resid0.clone()
+        prepared = ops.linear_into_stream(o, w_o, resid, hint)
+        assert ops._unmerged is None
+        return o, resid, prepared
+
+    o_ref, resid_ref, prep_ref = run(False)
+    o_new, resid_new, prep_new = run(True)
+    assert prep_ref is not None and prep_new is not None
+    assert torch.equal(resid_new, resid_ref)
+    assert torch.equal(prep_new.rows, prep_ref.rows)
+    assert torch.equal(prep_new.sumsq, prep_ref.sumsq)
+    # deferred, then met by another call: merged first, the same attention output
+    mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
+                       cache.k_pages.clone(), cache.v_pages.clone())
+    o = ops.attend(qkv, batch, table, mine, True, defer_merge=True, **kw).view(T, nq * hd)
+    y = ops.linear(o, w_o, dtype)
+    assert ops._unmerged is None
+    assert torch.equal(o, o_ref)
+    assert torch.equal(y, ops.linear(o_ref, w_o, dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
     """One key among hundreds, at a page's edge, is made to dominate: the output must be

@@ -32,6 +32,8 @@ struct AttentionDecodeArgs {
   const float* sin;
   float eps;
   int kv_in_row;            // nkv: the row brings k and v, written to the cache here; 0: q only
+  int defer_merge;          // 1: with more than one split, leave the partial results unmerged
+                            // (ts_gemm_tail_merged_bf16 or ts_attention_merge takes them)
 };
 
 int launch_attention_merge(const AttentionMfmaArgs& args, hipStream_t stream);
@@ -357,7 +359,7 @@ static int launch_decode(const AttentionDecodeArgs& args, hipStream_t stream) {
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
   }
-  if (m.num_splits > 1) return launch_attention_merge(m, stream);
+  if (m.num_splits > 1 && !args.defer_merge) return launch_attention_merge(m, stream);
   return 0;
 }
 

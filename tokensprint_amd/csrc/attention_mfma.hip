@@ -250,6 +250,16 @@ int launch_attention_merge(const AttentionMfmaArgs& args, hipStream_t stream) {
   return 0;
 }
 
+// The merge of a decode step's key splits that ts_attention_decode was told to leave.
+extern "C" int ts_attention_merge(const AttentionMfmaArgs* p, hipStream_t stream) {
+  const AttentionMfmaArgs& args = *p;
+  if (args.num_tiles <= 0 || args.num_splits <= 1) return 0;
+  if (!args.partial_o || !args.partial_ml) TS_FAIL("attention_merge: no partial results");
+  if (launch_attention_merge(args, stream)) return -1;
+  TS_CHECK_LAUNCH("attention_merge");
+  return 0;
+}
+
 extern "C" int ts_attention_mfma_chunk() { return kChunk; }
 
 int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who) {

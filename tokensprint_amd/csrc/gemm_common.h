@@ -55,6 +55,13 @@ struct DirectArgs {
   // root mean square that the slices of sums of squares give
   const float* sumsq;       // [parts][M]
   int parts;
+  // merged form (merge_o set; tail form, at most 16 rows): A is not stored either but is a
+  // decode step's attention output still lying in the partial sums of its key splits, as
+  // the attention kernels leave them for attention_merge; K = heads * merge_hd
+  const float* merge_o;     // [items, merge_splits, 16, merge_hd]
+  const float* merge_ml;    // [items, merge_splits, 16, 2]: row maximum (log2 units), sum
+  const int* merge_pos;     // [M]: position of each row's token
+  int merge_splits, merge_nkv, merge_group, merge_hd, merge_window, merge_chunk;
 };
 
 // Launches it; `norm` (the fused form) takes at most 16 rows.  Returns 0 or -1 with the

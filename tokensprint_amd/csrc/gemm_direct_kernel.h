@@ -30,9 +30,10 @@ __device__ __forceinline__ bf16x8 row_down_by(bf16x8 v, int n) {
 }
 
 template <int MT, int WK, typename TC, bool PAIR, bool NORM, int S, int PD, bool SCALED = false,
-          bool TAIL = false, int CW = 16, int AR = 16>
+          bool TAIL = false, int CW = 16, int AR = 16, bool MERGE = false>
 __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   static_assert(!NORM || MT == 1, "the fused form holds one tile of rows");
+  static_assert(!MERGE || (TAIL && MT == 1), "the merged form: a tail product of one tile of rows");
   // Packed operands.  A compute unit takes a wave's 16-byte load in about 28 cycles
   // whatever its lanes ask for, and that rate, not the bytes, bounds these products.  An
   // operand with fewer than 16 rows (AR rows of A that exist, CW rows of W that this
@@ -135,15 +136,25 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
     bf16x8 d[NORM ? S : 1];
     f32x4 nw[NORM ? S : 1][2];
   };
-  auto load = [&](Step& st, int kb) {
+  // merged form: the rows of A, merged out of the key splits' partial sums into LDS by
+  // the whole workgroup before the K loop; a row is K / 8 pieces and one of padding, so
+  // that the same piece of the 16 rows lies in 16 different banks
+  extern __shared__ __attribute__((aligned(16))) unsigned char merged_rows[];
+  const int row_pieces = K / 8 + 1;
+  const bf16x8* a_row = (const bf16x8*)merged_rows + min(m_base + r % AR, M - 1) * row_pieces +
+                        (g * kLane + (r / AR) * 8) / 8;
+  auto load = [&](Step& st, int kb, bool of_w = true, bool of_a = true) {
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      if (s % GW == 0) {
+      if (s % GW == 0 && of_w) {
 #pragma unroll
         for (int w = 0; w < NW; ++w)
           st.w[w][s / GW] = *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8);
       }
-      if constexpr (NORM) {
+      if (!of_a) continue;
+      if constexpr (MERGE) {
+        if (s % GA == 0) st.x[0][s / GA] = a_row[(kb + s * 8) / 8];
+      } else if constexpr (NORM) {
         const float* rp = a.resid_in + a_off[0] + kb + s * 8;
         st.rs[s][0] = *(const f32x4*)rp;
         st.rs[s][1] = *(const f32x4*)(rp + 4);
@@ -171,7 +182,10 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
         for (int w = 0; w < NW; ++w)
           st.w[w][s / GW] = ok_w ? *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8) : zero;
       }
-      if constexpr (NORM) {
+      if constexpr (MERGE) {
+        if (s % GA == 0)
+          st.x[0][s / GA] = kb + g * kLane + (s + r / AR) * 8 < K ? a_row[(kb + s * 8) / 8] : zero;
+      } else if constexpr (NORM) {
         const float* rp = a.resid_in + a_off[0] + kb + s * 8;
         st.rs[s][0] = ok ? *(const f32x4*)rp : fzero;
         st.rs[s][1] = ok ? *(const f32x4*)(rp + 4) : fzero;
@@ -226,6 +240,76 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   const int kb0 = wk * kStep;
   Step st[PD];
   int kb = kb0;
+  if constexpr (MERGE) {
+    // The first steps' rows of W are asked for, then every thread merges pieces of eight
+    // elements of A (the arithmetic of attention_merge, split by split in groups of
+    // eight, so the rows are bit for bit what that kernel would have stored), then the
+    // K loop runs with A out of LDS.
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+      if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride, true, false);
+    const int hd = a.merge_hd, splits = a.merge_splits, grp = a.merge_group;
+    const int head_blocks = (grp + 15) / 16;
+    const int pieces = K / 8;
+    bf16x8* rows = (bf16x8*)merged_rows;
+    for (int idx = threadIdx.x; idx < M * pieces; idx += WK * kWave) {
+      const int m = idx / pieces, p8 = idx % pieces;
+      const int head = p8 * 8 / hd, d = p8 * 8 % hd;
+      const int kvh = head / grp, hh = head % grp;
+      const int64_t base = ((int64_t)((m * a.merge_nkv + kvh) * head_blocks + hh / 16) * splits) * 16 + hh % 16;
+      const int pos = a.merge_pos[m];
+      const int lo = a.merge_window > 0 ? max(0, pos - a.merge_window + 1) : 0;
+      const int nchunks = pos / a.merge_chunk - lo / a.merge_chunk + 1;
+      const int per = (nchunks - 1 + splits) / splits;
+      const int used = min(splits, (nchunks + per - 1) / per);
+      float mx = -INFINITY, sum = 0.f, o[8] = {};
+      for (int s0 = 0; s0 == 0 || s0 < used; s0 += 8) {
+        float ms[8], ls[8];
+        f32x4 lo4[8], hi4[8];
+        // (the first eight splits are asked for without waiting for the position, which
+        // says how many hold keys at all; an empty one says so itself.  Later ones only
+        // if they hold keys: every workgroup merges all rows.)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t slot = base + (int64_t)min(s0 + j, splits - 1) * 16;
+          const bool holds = s0 == 0 ? j < splits : s0 + j < used;
+          ms[j] = holds ? a.merge_ml[slot * 2] : -INFINITY;
+          ls[j] = holds ? a.merge_ml[slot * 2 + 1] : 0.f;
+          lo4[j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d) : fzero;
+          hi4[j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d + 4) : fzero;
+        }
+        float mg = mx;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mg = (s0 + j < splits) ? fmaxf(mg, ms[j]) : mg;
+        if (mg == -INFINITY) continue;
+        const float keep = __builtin_amdgcn_exp2f(mx - mg);
+        sum *= keep;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] *= keep;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const bool live = s0 + j < splits && ms[j] != -INFINITY;
+          const float w = live ? __builtin_amdgcn_exp2f(ms[j] - mg) : 0.f;
+          sum += live ? ls[j] * w : 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            o[i] += live ? lo4[j][i] * w : 0.f;
+            o[4 + i] += live ? hi4[j][i] * w : 0.f;
+          }
+        }
+        mx = mg;
+      }
+      const float inv = sum > 0.f ? 1.f / sum : 0.f;
+      bf16x8 out;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[i] = (bf16_t)(o[i] * inv);
+      rows[m * row_pieces + p8] = out;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < PD; ++p)
+      if (kb0 + p * stride < kfull) load(st[p], kb0 + p * stride, false, true);
+  } else
   // (measured: with one workgroup to a compute unit the waits of the plain loop below,
   // which let all of a round's loads land before its products, serve better)
   if (kb0 + (2 * PD - 1) * stride < kfull && gridDim.x * gridDim.y >= 512) {
@@ -399,6 +483,23 @@ static inline void launch(const DirectArgs& a, hipStream_t stream) {
                      grid, dim3(WK * kWave), 0, stream, a);
 }
 
+// The merged tail form: dynamic LDS for the rows of A.  Returns false if the device
+// refuses that much.
+template <int WK, int CW, int AR>
+static inline bool launch_merged(const DirectArgs& a, hipStream_t stream) {
+  auto kernel = gemm_direct_kernel<1, WK, bf16_t, false, false, 4, 4, false, true, CW, AR, true>;
+  const size_t lds = (size_t)AR * (a.K / 8 + 1) * 16;
+  static size_t raised = 48 * 1024;      // per instantiation
+  if (lds > raised) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return false;
+    raised = lds;
+  }
+  hipLaunchKernelGGL(kernel, dim3((a.N + CW - 1) / CW, 1), dim3(WK * kWave), lds, stream, a);
+  return true;
+}
+
 
 // Tiles of 16 rows a workgroup holds, columns it owns and rows of A a load instruction is
 // packed for: the rules of gemm_direct.hip.
@@ -409,6 +510,7 @@ static inline int gemm_direct_packed_rows(int M) { return M <= 4 ? 4 : M <= 8 ? 
 // The forms' dispatchers, one per translation unit.
 int gemm_direct_plain(const DirectArgs& a, int c_type, hipStream_t stream);
 int gemm_direct_tail(const DirectArgs& a, hipStream_t stream);
+int gemm_direct_merged(const DirectArgs& a, hipStream_t stream);
 int gemm_direct_scaled(const DirectArgs& a, int c_type, bool pair, hipStream_t stream);
 int gemm_direct_pair(const DirectArgs& a, hipStream_t stream);
 int gemm_direct_norm(const DirectArgs& a, int c_type, bool pair, hipStream_t stream);

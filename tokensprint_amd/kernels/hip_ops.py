@@ -62,7 +62,7 @@ class AttentionDecodeArgs(Structure):
     _fields_ = [
         ("m", AttentionMfmaArgs), ("qkv", c_void_p), ("q_weight", c_void_p),
         ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("eps", c_float),
-        ("kv_in_row", c_int),
+        ("kv_in_row", c_int), ("defer_merge", c_int),
     ]
 
 
@@ -82,6 +82,16 @@ def _ptr(t: torch.Tensor | None):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
 
+class _UnmergedAttention:
+    """A decode step's attention output that still lies in the partial results of its key
+    splits: `out` is where the merge would put it."""
+
+    def __init__(self, out, args, partial_o, partial_ml, positions, window):
+        self.out, self.args = out, args                      # args: AttentionMfmaArgs
+        self.partial_o, self.partial_ml = partial_o, partial_ml
+        self.positions, self.window = positions, window
+
+
 class HipOps:
     name = "hip-gfx950"
 
@@ -99,6 +109,8 @@ class HipOps:
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
         self._timed_plans = False
+        self._unmerged = None          # an attention output whose merge was deferred
+        self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
 
     # ------------------------------------------------------------ helpers
     def _stream(self):
@@ -112,6 +124,8 @@ class HipOps:
     def _check(self, name, t, dtype=None, shape=None, ndim=None):
         # (written for the case that all is well, which is every call of a working engine:
         # this runs several times before every kernel)
+        if self._unmerged is not None and self._is_unmerged(t):
+            self._merge_now()
         try:
             ok = t.device == self.device and t.is_contiguous()
         except AttributeError:
@@ -137,6 +151,24 @@ class HipOps:
         raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
 
     _FLOATS = (torch.float32, torch.bfloat16)
+
+    # ------------------------------------------------------------ deferred merge
+    # A decode step's attention whose keys were split over workgroups ends in a merge of the
+    # splits' partial results.  `attend(defer_merge=True)` leaves that merge undone and
+    # remembers it; if the tensor it returned is next handed to `linear_into_stream` (the
+    # output projection in its tail form), that product's kernel merges the rows itself and
+    # a layer has one dependent kernel less.  Any other call of this provider that is given
+    # the tensor runs the merge first, so a caller sees nothing of this as long as the
+    # tensor goes nowhere but into this provider's calls (what `defer_merge` promises).
+    def _is_unmerged(self, t) -> bool:
+        try:
+            return t.data_ptr() == self._unmerged.out.data_ptr()
+        except AttributeError:
+            return False
+
+    def _merge_now(self) -> None:
+        pending, self._unmerged = self._unmerged, None
+        self._call(self.lib.ts_attention_merge, byref(pending.args), self._stream())
 
     # ------------------------------------------------------------ rows
     def embed(self, table, token_ids):
@@ -316,6 +348,11 @@ class HipOps:
         if hint is None or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or hint.weight.dtype != torch.bfloat16:
             return None
+        unmerged = self._unmerged if self._unmerged is not None and self._is_unmerged(x) else None
+        if unmerged is not None:
+            prepared = self._merged_into_stream(unmerged, x, weight, resid, hint)
+            if prepared is not None:
+                return prepared
         self._check("x", x, torch.bfloat16, ndim=2)
         self._check("weight", weight, torch.bfloat16, ndim=2)
         M, K = x.shape
@@ -335,6 +372,36 @@ class HipOps:
         sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_gemm_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
                    _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, self._stream())
+        return PreparedRows(rows, sumsq, hint)
+
+    def _merged_into_stream(self, unmerged, x, weight, resid, hint):
+        """`linear_into_stream` over an attention output that is still unmerged: one kernel
+        merges the rows and multiplies, if it takes the sizes; else None, nothing done."""
+        a = unmerged.args.base
+        M, K = x.shape
+        N = weight.shape[0]
+        if K != a.nq * a.hd or weight.shape[1] != K or M != a.num_tokens \
+                or not x.is_contiguous() or hint.weight.shape[1] != N \
+                or M > self.merged_rows:
+            return None
+        next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
+        parts = self.lib.ts_gemm_tail_parts(M, N)
+        if self._library_rows(M, N, K) or self._library_rows(M, next_n, N) \
+                or self.lib.ts_gemm_tail_merged_fits(M, N, a.nq, a.hd) != 1 \
+                or self.lib.ts_gemm_scaled_fits(M, next_n, N, int(hint.silu_mul), parts) != 1:
+            return None
+        self._unmerged = None
+        self._check("weight", weight, torch.bfloat16, ndim=2)
+        self._check("resid", resid, torch.float32, shape=(M, N))
+        self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
+        rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
+        sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
+        self._call(self.lib.ts_gemm_tail_merged_bf16, _ptr(unmerged.partial_o),
+                   _ptr(unmerged.partial_ml), _ptr(unmerged.positions),
+                   unmerged.args.num_splits, a.nq, a.nkv, a.hd,
+                   0 if unmerged.window is None else int(unmerged.window), _ptr(weight),
+                   _ptr(resid), _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N,
+                   self._stream())
         return PreparedRows(rows, sumsq, hint)
 
     def _prepared_linear(self, resid, prepared, norm_weight, eps, weight, out_dtype, silu_mul):
@@ -548,7 +615,8 @@ class HipOps:
         return out
 
     def attend(self, qkv, batch, table, cache, write_cache, *, num_heads, num_kv_heads,
-               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window):
+               kv_in_row, head_dim, q_weight, k_weight, eps, cos_sin, scale, window,
+               defer_merge=False):
         """Everything between the q/k/v projection and the output projection: per-head
         norm of q and k, rotation, the write of k and v into `cache` (if `write_cache`;
         the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
@@ -582,11 +650,16 @@ class HipOps:
         d = AttentionDecodeArgs()
         d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
         d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
-        self._attention_decode(a, batch, num_heads // num_kv_heads, d)
+        if self._unmerged is not None:      # one that nobody took: its tensor is dead
+            self._unmerged = None
+        self._attention_decode(a, batch, num_heads // num_kv_heads, d, out if defer_merge else None,
+                               window)
         return out
 
-    def _attention_decode(self, a, batch, group, d=None):
-        """One token per entry: workgroups per (entry, key/value head, share of the keys)."""
+    def _attention_decode(self, a, batch, group, d=None, defer_out=None, window=None):
+        """One token per entry: workgroups per (entry, key/value head, share of the keys).
+        `defer_out`: the output tensor, if the merge of the splits is to be left undone
+        and remembered (see `_is_unmerged`)."""
         d = d or AttentionDecodeArgs()
         m = d.m
         m.base = a
@@ -602,7 +675,12 @@ class HipOps:
             pml = torch.empty(items * m.num_splits * 16 * 2, dtype=torch.float32,
                               device=self.device)
             m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
+            if defer_out is not None and batch.num_entries <= self.merged_rows:
+                d.defer_merge = 1
         self._call(self.lib.ts_attention_decode, byref(d), self._stream())
+        if d.defer_merge:
+            kept = AttentionMfmaArgs.from_buffer_copy(m)
+            self._unmerged = _UnmergedAttention(defer_out, kept, po, pml, batch.positions, window)
 
     # Workgroups (entries x key/value heads) up to which a decode step takes the decode
     # kernel; with more, the chip is full anyway and the smaller workgroups of the general

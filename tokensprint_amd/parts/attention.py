@@ -100,7 +100,10 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 qkv, batch, table, cache, write_cache, num_heads=self.nq,
                 num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
-                cos_sin=tables, scale=self.scale, window=self.window)
+                cos_sin=tables, scale=self.scale, window=self.window,
+                # the result goes nowhere but into the output projection, a call of the
+                # same provider, which may then finish attention's last stage itself
+                defer_merge=True)
         else:
             # the encoding has no rotary table: norm only, let it encode, then store
             q, k, v = ops.qk_norm_split(
