@@ -252,59 +252,90 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
     const int head_blocks = (grp + 15) / 16;
     const int pieces = K / 8;
     bf16x8* rows = (bf16x8*)merged_rows;
-    for (int idx = threadIdx.x; idx < M * pieces; idx += WK * kWave) {
-      const int m = idx / pieces, p8 = idx % pieces;
-      const int head = p8 * 8 / hd, d = p8 * 8 % hd;
-      const int kvh = head / grp, hh = head % grp;
-      const int64_t base = ((int64_t)((m * a.merge_nkv + kvh) * head_blocks + hh / 16) * splits) * 16 + hh % 16;
-      const int pos = a.merge_pos[m];
-      const int lo = a.merge_window > 0 ? max(0, pos - a.merge_window + 1) : 0;
-      const int nchunks = pos / a.merge_chunk - lo / a.merge_chunk + 1;
-      const int per = (nchunks - 1 + splits) / splits;
-      const int used = min(splits, (nchunks + per - 1) / per);
-      float mx = -INFINITY, sum = 0.f, o[8] = {};
-      for (int s0 = 0; s0 == 0 || s0 < used; s0 += 8) {
-        float ms[8], ls[8];
-        f32x4 lo4[8], hi4[8];
-        // (the first eight splits are asked for without waiting for the position, which
-        // says how many hold keys at all; an empty one says so itself.  Later ones only
-        // if they hold keys: every workgroup merges all rows.)
+    // U pieces of a thread at a time, the loads of all of them asked for before the first
+    // is used (a piece after the other would cost a trip to memory each), in groups of G
+    // splits: few splits (decode steps of several rows) take four pieces of up to four
+    // splits, many (one or two rows) a piece of eight splits at a time.
+    auto merge_pieces = [&](auto group_size, auto at_a_time) {
+      constexpr int G = decltype(group_size)::value, U = decltype(at_a_time)::value;
+      constexpr int kThreads = WK * kWave;
+      for (int idx0 = threadIdx.x; idx0 < M * pieces; idx0 += U * kThreads) {
+        int64_t base[U];
+        int used[U], d[U];
+        float ms[U][G], ls[U][G];
+        f32x4 lo4[U][G], hi4[U][G];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int64_t slot = base + (int64_t)min(s0 + j, splits - 1) * 16;
-          const bool holds = s0 == 0 ? j < splits : s0 + j < used;
-          ms[j] = holds ? a.merge_ml[slot * 2] : -INFINITY;
-          ls[j] = holds ? a.merge_ml[slot * 2 + 1] : 0.f;
-          lo4[j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d) : fzero;
-          hi4[j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d + 4) : fzero;
-        }
-        float mg = mx;
+        for (int u = 0; u < U; ++u) {
+          const int idx = min(idx0 + u * kThreads, M * pieces - 1);     // past the end: the last again
+          const int m = idx / pieces, p8 = idx % pieces;
+          const int head = p8 * 8 / hd;
+          d[u] = p8 * 8 % hd;
+          const int kvh = head / grp, hh = head % grp;
+          base[u] = ((int64_t)((m * a.merge_nkv + kvh) * head_blocks + hh / 16) * splits) * 16 + hh % 16;
+          const int pos = a.merge_pos[m];
+          const int lo = a.merge_window > 0 ? max(0, pos - a.merge_window + 1) : 0;
+          const int nchunks = pos / a.merge_chunk - lo / a.merge_chunk + 1;
+          const int per = (nchunks - 1 + splits) / splits;
+          used[u] = min(splits, (nchunks + per - 1) / per);
+          // (the first group is asked for without waiting for the position, which says
+          // how many splits hold keys at all; an empty one says so itself)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mg = (s0 + j < splits) ? fmaxf(mg, ms[j]) : mg;
-        if (mg == -INFINITY) continue;
-        const float keep = __builtin_amdgcn_exp2f(mx - mg);
-        sum *= keep;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] *= keep;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const bool live = s0 + j < splits && ms[j] != -INFINITY;
-          const float w = live ? __builtin_amdgcn_exp2f(ms[j] - mg) : 0.f;
-          sum += live ? ls[j] * w : 0.f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            o[i] += live ? lo4[j][i] * w : 0.f;
-            o[4 + i] += live ? hi4[j][i] * w : 0.f;
+          for (int j = 0; j < G; ++j) {
+            const int64_t slot = base[u] + (int64_t)min(j, splits - 1) * 16;
+            const bool holds = j < splits;
+            ms[u][j] = holds ? a.merge_ml[slot * 2] : -INFINITY;
+            ls[u][j] = holds ? a.merge_ml[slot * 2 + 1] : 0.f;
+            lo4[u][j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d[u]) : fzero;
+            hi4[u][j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d[u] + 4) : fzero;
           }
         }
-        mx = mg;
-      }
-      const float inv = sum > 0.f ? 1.f / sum : 0.f;
-      bf16x8 out;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) out[i] = (bf16_t)(o[i] * inv);
-      rows[m * row_pieces + p8] = out;
-    }
+        for (int u = 0; u < U; ++u) {
+          float mx = -INFINITY, sum = 0.f, o[8] = {};
+          for (int s0 = 0; s0 == 0 || s0 < used[u]; s0 += G) {
+            if (s0 > 0) {      // later groups only if they hold keys: every workgroup merges all rows
+#pragma unroll
+              for (int j = 0; j < G; ++j) {
+                const int64_t slot = base[u] + (int64_t)min(s0 + j, splits - 1) * 16;
+                const bool holds = s0 + j < used[u];
+                ms[u][j] = holds ? a.merge_ml[slot * 2] : -INFINITY;
+                ls[u][j] = holds ? a.merge_ml[slot * 2 + 1] : 0.f;
+                lo4[u][j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d[u]) : fzero;
+                hi4[u][j] = holds ? *(const f32x4*)(a.merge_o + slot * hd + d[u] + 4) : fzero;
+              }
+            }
+            float mg = mx;
+#pragma unroll
+            for (int j = 0; j < G; ++j) mg = (s0 + j < splits) ? fmaxf(mg, ms[u][j]) : mg;
+            if (mg == -INFINITY) continue;
+            const float keep = __builtin_amdgcn_exp2f(mx - mg);
+            sum *= keep;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] *= keep;
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+              const bool live = s0 + j < splits && ms[u][j] != -INFINITY;
+              const float w = live ? __builtin_amdgcn_exp2f(ms[u][j] - mg) : 0.f;
+              sum += live ? ls[u][j] * w : 0.f;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                o[i] += live ? lo4[u][j][i] * w : 0.f;
+                o[4 + i] += live ? hi4[u][j][i] * w : 0.f;
+              }
+            }
+            mx = mg;
+          }
+          const float inv = sum > 0.f ? 1.f / sum : 0.f;
+          bf16x8 out;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) out[i] = (bf16_t)(o[i] * inv);
+          const int idx = idx0 + u * kThreads;
+          if (idx < M * pieces) rows[(idx / pieces) * row_pieces + idx % pieces] = out;
+        }
+      }
+    };
+    if (splits <= 4) merge_pieces(std::integral_constant<int, 4>{}, std::integral_constant<int, 4>{});
+    else merge_pieces(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{});
     __syncthreads();
 #pragma unroll
     for (int p = 0; p < PD; ++p)
