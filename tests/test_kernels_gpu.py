@@ -578,6 +578,36 @@ def attend_decode_case(ops, gpu_device, dtype, nq, nkv, hd, page, window, spans)
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("nq,nkv,hd,spans", [
+    (16, 8, 128, [(5000, 1), (2047, 1), (3, 1), (2049, 1), (130, 1)]),
+    (32, 8, 128, [(900, 1)] * 7), (64, 8, 128, [(4000, 1), (129, 1)]),
+    (12, 2, 64, [(3000, 1), (0, 1), (257, 1)]), (40, 1, 96, [(1500, 1), (700, 1)])])
+@pytest.mark.parametrize("window", [None, 1000])
+def test_decode_kernel_merges_its_key_splits_as_the_merge_kernel_does(ops, gpu_device, monkeypatch,
+                                                                      nq, nkv, hd, spans, window):
+    """The workgroup of an item that finishes last merges the item's key splits; the result
+    is, bit for bit, the merge kernel's, time after time (the arrival counts are left at
+    zero), with splits that hold no keys beside full ones."""
+    dtype, page = torch.bfloat16, 16
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=spans, seed=71)
+    assert ops._decode_splits(len(spans) * nkv * -(-(nq // nkv) // 16), batch.max_ctx_len) > 1
+    qkv = rand((batch.num_tokens, (nq + 2 * nkv) * hd), dtype, gpu_device, 72)
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 73)
+    angles = torch.outer(torch.arange(5100, dtype=torch.float32),
+                         1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, q_weight=wq, k_weight=wq, eps=1e-6,
+              cos_sin=cos_sin, scale=hd ** -0.5, window=window, kv_in_row=nkv)
+    assert ops.fold_merge
+    folded = [ops.attend(qkv, batch, table, cache, True, **kw).clone() for _ in range(3)]
+    assert int(ops._arrivals.abs().sum()) == 0
+    monkeypatch.setattr(ops, "fold_merge", False)
+    apart = ops.attend(qkv, batch, table, cache, True, **kw)
+    for out in folded:
+        assert torch.equal(out, apart)
+
+
 @pytest.mark.parametrize("window", [None, 1000])
 @pytest.mark.parametrize("fused", [True, False])
 def test_attend_decode_long_contexts_split_and_merge(ops, gpu_device, window, fused):

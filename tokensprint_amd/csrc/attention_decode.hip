@@ -6,7 +6,7 @@
 // waves take every NW-th block of 32 keys with the loads and arithmetic of
 // attention_core.h and merge in LDS, so up to a few thousand keys cost one launch and no
 // partial results in memory; longer contexts are split over workgroups and merged by
-// attention_merge.
+// attention_merge, or by the workgroup of the item that finishes last (below).
 //
 // Fused form (FUSED): what lies between the q/k/v projection and attention happens here
 // as well, so a decode layer needs no kernel for it.  Every wave reads its query rows
@@ -34,6 +34,9 @@ struct AttentionDecodeArgs {
   int kv_in_row;            // nkv: the row brings k and v, written to the cache here; 0: q only
   int defer_merge;          // 1: with more than one split, leave the partial results unmerged
                             // (ts_gemm_tail_merged_bf16 or ts_attention_merge takes them)
+  unsigned* arrivals;       // [items] zeros, or null.  Given (and the merge not deferred), the
+                            // workgroup of an item that finishes last merges the splits itself
+                            // and leaves the item's count at zero: no merge kernel
 };
 
 int launch_attention_merge(const AttentionMfmaArgs& args, hipStream_t stream);
@@ -89,6 +92,75 @@ __device__ __forceinline__ void prepare_head(bf16x8 (&v)[HD / 32], bool live, bo
 #pragma unroll
     for (int j = 0; j < 8; ++j) o[j] = (bf16_t)x[j];
     v[s] = live ? o : zero8;
+  }
+}
+
+// A float32 to memory, and back, at device scope without ordering: such accesses pass the
+// caches that another XCD does not share.
+__device__ __forceinline__ void store_past_caches(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_past_caches(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The merge of attention_merge_kernel (same order, same arithmetic per element, so the same
+// bits) by the THREADS threads of one workgroup, over the `used` first splits of one item:
+// slot (first_slot + split * 16 + row) holds a row's statistics and HD partial sums.  A
+// thread takes two elements at a time and asks for all of a group of eight splits before it
+// uses the first.
+template <int HD, int THREADS>
+__device__ __forceinline__ void merge_splits_here(const float* partial_o, const float* partial_ml,
+                                                  int64_t first_slot, int used, int rows, bf16_t* out) {
+  constexpr int kGroup = 8, E = 2;
+  const int count = rows * HD;
+  for (int e0 = threadIdx.x; e0 < count; e0 += E * THREADS) {
+    int row[E], d[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const int e = min(e0 + k * THREADS, count - 1);    // past the end: the last again, not stored
+      row[k] = e / HD;
+      d[k] = e % HD;
+    }
+    float M[E], L[E], acc[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) { M[k] = -INFINITY; L[k] = 0.f; acc[k] = 0.f; }
+    for (int s0 = 0; s0 < used; s0 += kGroup) {
+      float ms[E][kGroup], ls[E][kGroup], part[E][kGroup];
+#pragma unroll
+      for (int j = 0; j < kGroup; ++j)
+#pragma unroll
+        for (int k = 0; k < E; ++k) {
+          const int64_t slot = first_slot + (int64_t)min(s0 + j, used - 1) * 16 + row[k];
+          ms[k][j] = load_past_caches(partial_ml + slot * 2);
+          ls[k][j] = load_past_caches(partial_ml + slot * 2 + 1);
+          part[k][j] = load_past_caches(partial_o + slot * HD + d[k]);
+        }
+#pragma unroll
+      for (int k = 0; k < E; ++k) {
+        float Mg = M[k];
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) Mg = (s0 + j < used) ? fmaxf(Mg, ms[k][j]) : Mg;
+        if (Mg == -INFINITY) continue;
+        const float keep = __builtin_amdgcn_exp2f(M[k] - Mg);
+        L[k] *= keep;
+        acc[k] *= keep;
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+          const bool live = s0 + j < used && ms[k][j] != -INFINITY;
+          const float w = live ? __builtin_amdgcn_exp2f(ms[k][j] - Mg) : 0.f;
+          L[k] += live ? ls[k][j] * w : 0.f;
+          acc[k] += live ? part[k][j] * w : 0.f;
+        }
+        M[k] = Mg;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      if (e0 + k * THREADS >= count) break;
+      const float inv = L[k] > 0.f ? 1.f / L[k] : 0.f;
+      out[(int64_t)row[k] * HD + d[k]] = (bf16_t)(acc[k] * inv);
+    }
   }
 }
 
@@ -282,47 +354,84 @@ __global__ __launch_bounds__(decode_waves<HD>() * kWave) void attention_decode_k
   for (int db = 0; db < DB; ++db) s_o[wave][db][lane] = o[db];
   __syncthreads();
   constexpr int kShare = (DB + NW - 1) / NW;         // blocks of 16 elements per wave
-  if (wave * kShare >= DB) return;
-  float M = -INFINITY;
-#pragma unroll
-  for (int w = 0; w < NW; ++w) M = fmaxf(M, s_ml[w][lane][0]);
-  float ww[NW];
-  l = 0.f;
-#pragma unroll
-  for (int w = 0; w < NW; ++w) {
-    const float mw = s_ml[w][lane][0];
-    // a wave that saw no key has m = -inf (and so has everyone if M is): weight 0
-    ww[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
-    l += s_ml[w][lane][1] * ww[w];
-  }
-  m = M;
-  // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  // Merge by the last to finish: the partial results go out past the caches (their readers
+  // may sit on another XCD, behind another L2), each wave waits until its own have been
+  // taken, the workgroup counts itself in at the item's counter, and the one that finds
+  // all the others there reads every split's result back the same way and merges them in
+  // the order and arithmetic of attention_merge.  Nothing here needs the caches written
+  // back or dropped, which is what release and acquire at device scope would cost.
+  const bool fold = ma.num_splits > 1 && !args.defer_merge && args.arrivals != nullptr;
+  const bool has_share = wave * kShare < DB;
+  if (!has_share && !fold) return;
   const int64_t slot = ((int64_t)item * ma.num_splits + split) * 16 + r;
+  if (has_share) {
+    float M = -INFINITY;
 #pragma unroll
-  for (int k = 0; k < kShare; ++k) {
-    const int db = wave * kShare + k;
-    if (db >= DB) break;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, s_ml[w][lane][0]);
+    float ww[NW];
+    l = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
-      const f32x4 ow = s_o[w][db][lane];
+      const float mw = s_ml[w][lane][0];
+      // a wave that saw no key has m = -inf (and so has everyone if M is): weight 0
+      ww[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+      l += s_ml[w][lane][1] * ww[w];
+    }
+    m = M;
+    // lane (r, g) holds O^T[d = db*16 + g*4 + i][row r]
+    const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] += ww[w] == 0.f ? 0.f : ow[i] * ww[w];   // never 0 * garbage
+    for (int k = 0; k < kShare; ++k) {
+      const int db = wave * kShare + k;
+      if (db >= DB) break;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const f32x4 ow = s_o[w][db][lane];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += ww[w] == 0.f ? 0.f : ow[i] * ww[w];   // never 0 * garbage
+      }
+      if (!row_ok) continue;
+      if (ma.num_splits == 1) {
+        bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv),
+                     (bf16_t)(acc[3] * inv)};
+        *(bf16x4*)((bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD + db * 16 + g * 4) = ov;
+      } else if (fold) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) store_past_caches(ma.partial_o + slot * HD + db * 16 + g * 4 + i, acc[i]);
+      } else {
+        *(f32x4*)(ma.partial_o + slot * HD + db * 16 + g * 4) = acc;
+      }
     }
-    if (!row_ok) continue;
-    if (ma.num_splits == 1) {
-      bf16x4 ov = {(bf16_t)(acc[0] * inv), (bf16_t)(acc[1] * inv), (bf16_t)(acc[2] * inv),
-                   (bf16_t)(acc[3] * inv)};
-      *(bf16x4*)((bf16_t*)a.out + ((int64_t)token * a.nq + head) * HD + db * 16 + g * 4) = ov;
-    } else {
-      *(f32x4*)(ma.partial_o + slot * HD + db * 16 + g * 4) = acc;
+    if (ma.num_splits > 1 && wave == 0 && g == 0) {
+      if (fold) {
+        store_past_caches(ma.partial_ml + slot * 2, m);
+        store_past_caches(ma.partial_ml + slot * 2 + 1, l);
+      } else {
+        ma.partial_ml[slot * 2] = m;
+        ma.partial_ml[slot * 2 + 1] = l;
+      }
     }
   }
-  if (ma.num_splits > 1 && wave == 0 && g == 0) {
-    ma.partial_ml[slot * 2] = m;
-    ma.partial_ml[slot * 2 + 1] = l;
-  }
+  if (!fold) return;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);                     // this wave's stores have been taken
+  __shared__ unsigned s_before;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    s_before = __hip_atomic_fetch_add(args.arrivals + item, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  // splits that hold chunks: the arithmetic of attention_merge; the others have returned
+  const int nchunks = c_last - c_first + 1;
+  const int used = min(ma.num_splits, (nchunks + per - 1) / per);
+  if ((int)s_before + 1 != used) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (threadIdx.x == 0)
+    __hip_atomic_store(args.arrivals + item, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const int rows = min(ma.rows_per_token, group - hb * 16);
+  bf16_t* out = (bf16_t*)a.out + ((int64_t)token * a.nq + kvh * group + hb * 16) * HD;
+  merge_splits_here<HD, NW * kWave>(ma.partial_o, ma.partial_ml, (int64_t)item * ma.num_splits * 16,
+                                    used, rows, out);
 }
 
 int ts_check_attention_mfma_args(const AttentionMfmaArgs& args, const char* who);
@@ -359,7 +468,7 @@ static int launch_decode(const AttentionDecodeArgs& args, hipStream_t stream) {
     }
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
   }
-  if (m.num_splits > 1 && !args.defer_merge) return launch_attention_merge(m, stream);
+  if (m.num_splits > 1 && !args.defer_merge && !args.arrivals) return launch_attention_merge(m, stream);
   return 0;
 }
 

@@ -31,9 +31,11 @@ extern "C" int ts_gemm_tail_merged_fits(int M, int N, int heads, int hd) {
 
 // Rows up to which it pays.  Every workgroup merges all rows, and what it reads for that
 // grows with the rows while the kernel it saves does not: measured in decode steps of
-// the 0.6B shape, a step is 6.4 % shorter at one row, 4.1 % at two, 1.2 % at three, the
-// same at four, 1 to 3 % longer from five to eight.
-extern "C" int ts_gemm_tail_merged_rows() { return 3; }
+// the 0.6B shape against a merge kernel of its own, a step is 6.4 % shorter at one row,
+// 4.1 % at two, 1.2 % at three, the same at four, 1 to 3 % longer from five to eight.
+// Against the decode kernel merging its splits itself (the item's last workgroup to
+// finish) it is 3 % ahead at one row, 1 % at two and 2 % behind at three.
+extern "C" int ts_gemm_tail_merged_rows() { return 2; }
 
 // ts_gemm_tail_bf16 with A = the attention output of a decode step of M tokens that
 // ts_attention_decode left unmerged (`defer_merge`): partial_o [M * nkv * ceil(group / 16),

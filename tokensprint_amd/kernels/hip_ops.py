@@ -62,7 +62,7 @@ class AttentionDecodeArgs(Structure):
     _fields_ = [
         ("m", AttentionMfmaArgs), ("qkv", c_void_p), ("q_weight", c_void_p),
         ("k_weight", c_void_p), ("cos", c_void_p), ("sin", c_void_p), ("eps", c_float),
-        ("kv_in_row", c_int), ("defer_merge", c_int),
+        ("kv_in_row", c_int), ("defer_merge", c_int), ("arrivals", c_void_p),
     ]
 
 
@@ -111,6 +111,11 @@ class HipOps:
         self._timed_plans = False
         self._unmerged = None          # an attention output whose merge was deferred
         self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
+        # Above those rows the decode kernel merges its key splits itself: the workgroups of
+        # an item count themselves in here and the last one merges.  The kernel leaves every
+        # count at zero, so one zeroed array serves every launch (of one stream).
+        self.fold_merge = True
+        self._arrivals = torch.zeros(4096, dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------ helpers
     def _stream(self):
@@ -677,6 +682,8 @@ class HipOps:
             m.partial_o, m.partial_ml = po.data_ptr(), pml.data_ptr()
             if defer_out is not None and batch.num_entries <= self.merged_rows:
                 d.defer_merge = 1
+            elif self.fold_merge and items <= self._arrivals.numel():
+                d.arrivals = self._arrivals.data_ptr()
         self._call(self.lib.ts_attention_decode, byref(d), self._stream())
         if d.defer_merge:
             kept = AttentionMfmaArgs.from_buffer_copy(m)
