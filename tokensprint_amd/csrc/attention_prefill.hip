@@ -466,21 +466,21 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
     // for into buffer `to`, which block j - 1 was read from.
     auto turn = [&](int j, int from, int to) {
       const int kb = kb_first + 32 * H * j;
-      if (j + 2 < mine) {
-        issue(j + 2, to);
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoads));    // all but the two youngest blocks
-      } else if (j + 1 < mine) {
-        __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-      }
+      // this wave's share of block j has arrived: at most block j + 1's loads are in flight
+      if (j + 1 < mine) __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
       // Every wave's share of block j is in LDS, and every wave is through with block
       // j - 1.  The bare barrier: __syncthreads would first wait for every load in flight,
-      // the two younger blocks' among them.  The empty statements keep the compiler from
+      // the younger block's among them.  The empty statements keep the compiler from
       // moving LDS reads across it.
       asm volatile("" ::: "memory");
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
+      // Only now may block j - 1's buffer be written: a wave that has nothing to do with a
+      // block (outside its tile's window, or past its tile's last row) runs ahead of the
+      // others by a whole turn, and loads sent for before the barrier could land while a
+      // slower wave still reads that buffer.
+      if (j + 2 < mine) issue(j + 2, to);
       if (j < mine && kb <= tile_last && kb + 31 >= tile_lo) {
         const Slots kcur = ring + from * kSlots, vcur = kcur + 2 * KS;
         KvBlock<HD> b;
