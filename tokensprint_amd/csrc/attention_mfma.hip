@@ -20,7 +20,7 @@
 // COOP = true: a workgroup per item; its four waves take every fourth 32-key block and
 // merge in LDS (few tiles: decode), so a short context costs one round of loads.
 template <int HD, bool COOP, bool PAGE16>
-__global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs args) {
+__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attention_mfma_kernel(AttentionMfmaArgs args) {
   constexpr int DB = HD / 16;
   const AttentionArgs& a = args.base;
   const int wave = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
@@ -76,16 +76,21 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(AttentionMfmaArgs a
   if (PAGE16) cur.start(key_begin);
 
   KvBlock<HD> A, B;
-  if (key_begin < key_end) load_kv_block<HD, PAGE16>(A, a, table, cur, kvh, key_begin, kStride, r, g);
+  // head sizes in whole 32-element slices on power-of-two pages take the blocks with
+  // 16-byte value loads (the keys of a block permuted over the score products' rows)
+  constexpr bool kWide = PAGE16 && HD % 32 == 0;
+  auto load_block = [&](KvBlock<HD>& b, int kb) {
+    if constexpr (kWide) load_kv_block_wide<HD>(b, a, cur, kvh, kb, kStride, r, g);
+    else load_kv_block<HD, PAGE16>(b, a, table, cur, kvh, kb, kStride, r, g);
+  };
+  if (key_begin < key_end) load_block(A, key_begin);
   for (int kb = key_begin; kb < key_end; kb += 2 * kStride) {
-    if (kb + kStride < key_end)
-      load_kv_block<HD, PAGE16>(B, a, table, cur, kvh, kb + kStride, kStride, r, g);
-    tile_update<HD>(t, A, kb, scale_log2, kb + 31 <= pos_first && kb >= lo_last, g);
+    if (kb + kStride < key_end) load_block(B, kb + kStride);
+    tile_update<HD, false, kWide>(t, A, kb, scale_log2, kb + 31 <= pos_first && kb >= lo_last, g);
     if (kb + kStride >= key_end) break;
-    if (kb + 2 * kStride < key_end)
-      load_kv_block<HD, PAGE16>(A, a, table, cur, kvh, kb + 2 * kStride, kStride, r, g);
-    tile_update<HD>(t, B, kb + kStride, scale_log2,
-                    kb + kStride + 31 <= pos_first && kb + kStride >= lo_last, g);
+    if (kb + 2 * kStride < key_end) load_block(A, kb + 2 * kStride);
+    tile_update<HD, false, kWide>(t, B, kb + kStride, scale_log2,
+                                  kb + kStride + 31 <= pos_first && kb + kStride >= lo_last, g);
   }
   f32x4 (&o)[DB] = t.o;
   float m = t.m, l = row_sum<HD>(t);
