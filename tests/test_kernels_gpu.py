@@ -600,7 +600,9 @@ def attend_decode_case(ops, gpu_device, dtype, nq, nkv, hd, page, window, spans)
 @pytest.mark.parametrize("nq,nkv,hd,spans", [
     (16, 8, 128, [(5000, 1), (2047, 1), (3, 1), (2049, 1), (130, 1)]),
     (32, 8, 128, [(900, 1)] * 7), (64, 8, 128, [(4000, 1), (129, 1)]),
-    (12, 2, 64, [(3000, 1), (0, 1), (257, 1)]), (40, 1, 96, [(1500, 1), (700, 1)])])
+    (12, 2, 64, [(3000, 1), (0, 1), (257, 1)]), (40, 1, 96, [(1500, 1), (700, 1)]),
+    (6, 3, 48, [(2100, 1), (127, 1), (640, 1)]), (10, 2, 80, [(900, 1), (1300, 1)]),
+    (4, 4, 256, [(1000, 1), (130, 1)])])
 @pytest.mark.parametrize("window", [None, 1000])
 def test_decode_kernel_merges_its_key_splits_as_the_merge_kernel_does(ops, gpu_device, monkeypatch,
                                                                       nq, nkv, hd, spans, window):
