@@ -209,3 +209,41 @@ def test_bfloat16_logits_of_the_generated_tokens(setup, gpu_device):
         for p, row in got.items():
             torch.testing.assert_close(row, ref[p], rtol=3e-2, atol=3e-2)
     assert runner.graphs                 # the single-token steps were replays
+
+
+def test_warm_up_chooses_who_multiplies_large_weights(setup, gpu_device, tmp_path, monkeypatch):
+    """With weights that count as large (here: all of them), the warm-up times a captured
+    decode step with the provider's own products of few rows and with the library's and
+    keeps one; under either choice the steps' logits are the plain ones.  (Weights written
+    in bfloat16: float32 ones stay float32 and never meet the library.)"""
+    from tokensprint_amd.engine import StepEntry
+    cfg, _, _, page, prompts, _ = setup
+    seed = 3
+    d = write_random_model(tmp_path / "model", cfg, seed, torch.bfloat16)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, torch.bfloat16, gpu_device)
+    ops = model.ctx.ops
+    monkeypatch.setattr(ops, "LARGE_WEIGHT", 1 << 8)
+    monkeypatch.setattr(ops, "_saw_large_weight", False)
+    monkeypatch.setattr(ops, "LIBRARY_ROWS_LARGE", type(ops).LIBRARY_ROWS_LARGE)
+    L = cfg["max_position_embeddings"]
+    engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L)
+    choices = ops.large_weight_choices()
+    assert choices and choices[0] in (9, 1) and set(choices) == {9, 1}
+    assert set(engine.runner.graphs) == set(engine.runner.buckets)     # the trials were dropped
+    for rows in (9, 1):
+        ops.set_large_weight_rows(rows)
+        runner = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L,
+                            warmup=False).runner
+        for prompt in prompts[:3]:
+            tokens = prompt + plain.greedy_generate(pcfg, w, prompt, 6)
+            ref = plain.forward_logits(pcfg, w, tokens)
+            rc = runner.manager.admit("r")
+            pos = 0
+            for n in [len(prompt)] + [1] * 6:
+                runner.manager.extend(rc, pos + n)
+                row = runner.step([StepEntry(rc, tokens[pos:pos + n], pos, [n - 1])])[0]
+                torch.testing.assert_close(row.float().cpu(), ref[pos + n - 1], rtol=3e-2, atol=3e-2)
+                pos += n
+            runner.manager.free(rc)
+        assert runner.graphs

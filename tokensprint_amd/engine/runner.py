@@ -9,6 +9,8 @@ left; portions of prompts and single decoded tokens may be mixed and cut anywher
 
 from __future__ import annotations
 
+import time
+
 import torch
 
 from tokensprint_amd.cache import CacheManager, CacheStorage, page_bytes
@@ -131,9 +133,35 @@ class ModelRunner:
         """Capture every decode bucket now, the largest first so that the smaller ones fit
         into the memory it took (engine/generation/model_runner.py:334,373-379 captures in
         that order for that reason).  Without this a bucket is captured at its first use."""
+        self._choose_large_weight_rows()
         for bucket in reversed(self.buckets):
             if bucket not in self.graphs:
                 self._capture(bucket)
+
+    def _choose_large_weight_rows(self) -> None:
+        """Where the kernel provider has a choice to offer for the products of few rows
+        with large weights (its own kernels or the vendor library's), take the one whose
+        captured decode step of the smallest bucket replays faster; the one in force stays
+        unless another is 3 % ahead."""
+        ops = self.model.ctx.ops
+        choices = getattr(ops, "large_weight_choices", lambda: ())()
+        if len(choices) < 2 or not self.buckets or self.graphs:
+            return
+        bucket, seconds = self.buckets[0], []
+        for rows in choices:
+            ops.set_large_weight_rows(rows)
+            graph = self._capture(bucket)[0]
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize(self.device)
+            start = time.perf_counter()
+            for _ in range(10):
+                graph.replay()
+            torch.cuda.synchronize(self.device)
+            seconds.append(time.perf_counter() - start)
+            del self.graphs[bucket], graph
+        best = min(range(len(choices)), key=lambda i: seconds[i])
+        ops.set_large_weight_rows(choices[best] if seconds[best] < 0.97 * seconds[0] else choices[0])
 
     def dummy_step(self, num_tokens: int, num_entries: int) -> int:
         """Run one step of `num_tokens` zero tokens in `num_entries` requests (fewer of

@@ -110,6 +110,7 @@ class HipOps:
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
         self._timed_plans = False
+        self._saw_large_weight = False
         self._unmerged = None          # an attention output whose merge was deferred
         self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
         # Above those rows the decode kernel merges its key splits itself: the workgroups of
@@ -327,14 +328,30 @@ class HipOps:
             return False
         return self._library_rows(x.shape[0], weight.shape[0], weight.shape[1])
 
+    def large_weight_choices(self):
+        """Row counts from which products with a large weight may go to the library, for the
+        warm-up to try in a captured decode step, the one in force first; empty while no such
+        weight has been met.  At the Qwen3-8B shapes the kernels here are ahead below nine
+        rows (a decode step of one row 3.61 against 4.07 ms), at the 32B shapes (a hidden
+        size of 5,120: 320 or 640 workgroups for 256 compute units, and a K that the loads'
+        steps divide less well) the library is, by 15 to 20 %, norm kernels and all."""
+        if not self._saw_large_weight:
+            return ()
+        return tuple(dict.fromkeys((self.LIBRARY_ROWS_LARGE, type(self).LIBRARY_ROWS_LARGE, 1)))
+
+    def set_large_weight_rows(self, rows: int) -> None:
+        self.LIBRARY_ROWS_LARGE = int(rows)
+
     def _library_rows(self, M, N, K):
         """Whether a bfloat16 product of M rows with a weight [N, K] is the library's."""
         if M >= self.LIBRARY_ROWS:
             return True
         if M >= self.LIBRARY_ROWS_HEAD and N >= self.HEAD_COLUMNS:
             return True
-        if M >= self.LIBRARY_ROWS_LARGE and N * K > self.LARGE_WEIGHT:
-            return True
+        if N * K > self.LARGE_WEIGHT:
+            self._saw_large_weight = True
+            if M >= self.LIBRARY_ROWS_LARGE:
+                return True
         return M >= self.LIBRARY_ROWS_WIDE and self.lib.ts_gemm_mfma_layout(N, K) == 2
 
     @staticmethod
