@@ -224,15 +224,16 @@ def test_warm_up_chooses_who_multiplies_large_weights(setup, gpu_device, tmp_pat
     _, model = load_model(d, torch.bfloat16, gpu_device)
     ops = model.ctx.ops
     monkeypatch.setattr(ops, "LARGE_WEIGHT", 1 << 8)
-    monkeypatch.setattr(ops, "_saw_large_weight", False)
-    monkeypatch.setattr(ops, "LIBRARY_ROWS_LARGE", type(ops).LIBRARY_ROWS_LARGE)
+    monkeypatch.setattr(ops, "_large_rows", {})
+    monkeypatch.setattr(ops, "_large_undecided", set())
     L = cfg["max_position_embeddings"]
     engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L)
-    choices = ops.large_weight_choices()
-    assert choices and choices[0] in (9, 1) and set(choices) == {9, 1}
+    chosen = dict(ops._large_rows)
+    assert chosen and len(set(chosen.values())) == 1 and set(chosen.values()) <= {9, 1}
+    assert ops.large_weight_choices() == ()          # every shape met has its choice
     assert set(engine.runner.graphs) == set(engine.runner.buckets)     # the trials were dropped
     for rows in (9, 1):
-        ops.set_large_weight_rows(rows)
+        monkeypatch.setattr(ops, "_large_rows", {shape: rows for shape in chosen})
         runner = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L,
                             warmup=False).runner
         for prompt in prompts[:3]:

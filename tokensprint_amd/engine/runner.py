@@ -149,7 +149,7 @@ class ModelRunner:
             return
         bucket, seconds = self.buckets[0], []
         for rows in choices:
-            ops.set_large_weight_rows(rows)
+            ops.try_large_weight_rows(rows)
             graph = self._capture(bucket)[0]
             for _ in range(3):
                 graph.replay()
@@ -161,7 +161,7 @@ class ModelRunner:
             seconds.append(time.perf_counter() - start)
             del self.graphs[bucket], graph
         best = min(range(len(choices)), key=lambda i: seconds[i])
-        ops.set_large_weight_rows(choices[best] if seconds[best] < 0.97 * seconds[0] else choices[0])
+        ops.keep_large_weight_rows(choices[best] if seconds[best] < 0.97 * seconds[0] else choices[0])
 
     def dummy_step(self, num_tokens: int, num_entries: int) -> int:
         """Run one step of `num_tokens` zero tokens in `num_entries` requests (fewer of

@@ -110,7 +110,9 @@ class HipOps:
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
         self._timed_plans = False
-        self._saw_large_weight = False
+        # products of few rows with large weights: ours or the library's, per weight shape
+        # (see large_weight_choices)
+        self._large_rows, self._large_undecided, self._large_trial = {}, set(), None
         self._unmerged = None          # an attention output whose merge was deferred
         self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
         # Above those rows the decode kernel merges its key splits itself: the workgroups of
@@ -330,17 +332,27 @@ class HipOps:
 
     def large_weight_choices(self):
         """Row counts from which products with a large weight may go to the library, for the
-        warm-up to try in a captured decode step, the one in force first; empty while no such
-        weight has been met.  At the Qwen3-8B shapes the kernels here are ahead below nine
-        rows (a decode step of one row 3.61 against 4.07 ms), at the 32B shapes (a hidden
-        size of 5,120: 320 or 640 workgroups for 256 compute units, and a K that the loads'
-        steps divide less well) the library is, by 15 to 20 %, norm kernels and all."""
-        if not self._saw_large_weight:
+        warm-up to try in a captured decode step, the default first; empty unless a large
+        weight of a shape that has no choice yet has been met.  At the Qwen3-8B shapes the
+        kernels here are ahead below nine rows (a decode step of one row 3.61 against
+        4.07 ms), at the 32B shapes (a hidden size of 5,120: 320 or 640 workgroups for 256
+        compute units, and a K that the loads' steps divide less well) the library is, by 15
+        to 20 %, norm kernels and all.  A choice is kept per weight shape (N, K), so that
+        models of other shapes in the same process get their own."""
+        if not self._large_undecided:
             return ()
-        return tuple(dict.fromkeys((self.LIBRARY_ROWS_LARGE, type(self).LIBRARY_ROWS_LARGE, 1)))
+        return (self.LIBRARY_ROWS_LARGE, 1)
 
-    def set_large_weight_rows(self, rows: int) -> None:
-        self.LIBRARY_ROWS_LARGE = int(rows)
+    def try_large_weight_rows(self, rows) -> None:
+        """For the shapes without a choice: `rows` for now (None: the default again)."""
+        self._large_trial = rows
+
+    def keep_large_weight_rows(self, rows: int) -> None:
+        """The shapes met so far without a choice get `rows` for good."""
+        for shape in self._large_undecided:
+            self._large_rows[shape] = int(rows)
+        self._large_undecided = set()
+        self._large_trial = None
 
     def _library_rows(self, M, N, K):
         """Whether a bfloat16 product of M rows with a weight [N, K] is the library's."""
@@ -349,8 +361,11 @@ class HipOps:
         if M >= self.LIBRARY_ROWS_HEAD and N >= self.HEAD_COLUMNS:
             return True
         if N * K > self.LARGE_WEIGHT:
-            self._saw_large_weight = True
-            if M >= self.LIBRARY_ROWS_LARGE:
+            rows = self._large_rows.get((N, K))
+            if rows is None:
+                self._large_undecided.add((N, K))
+                rows = self.LIBRARY_ROWS_LARGE if self._large_trial is None else self._large_trial
+            if M >= rows:
                 return True
         return M >= self.LIBRARY_ROWS_WIDE and self.lib.ts_gemm_mfma_layout(N, K) == 2
 
