@@ -141,16 +141,17 @@ class ModelRunner:
     def _choose_large_weight_rows(self) -> None:
         """Where the kernel provider has a choice to offer for the products of few rows
         with large weights (its own kernels or the vendor library's), take the one whose
-        captured decode step of the smallest bucket replays faster; the one in force stays
-        unless another is 3 % ahead."""
+        captured decode step of the smallest bucket replays faster; the default stays
+        unless another is 3 % ahead.  The default's step is captured first: running it is
+        how the provider meets the shapes, and if the default stays it is that bucket's
+        graph."""
         ops = self.model.ctx.ops
-        choices = getattr(ops, "large_weight_choices", lambda: ())()
-        if len(choices) < 2 or not self.buckets or self.graphs:
+        offers = getattr(ops, "large_weight_choices", None)
+        if offers is None or not self.buckets or self.graphs:
             return
-        bucket, seconds = self.buckets[0], []
-        for rows in choices:
-            ops.try_large_weight_rows(rows)
-            graph = self._capture(bucket)[0]
+        bucket = self.buckets[0]
+
+        def seconds(graph):
             for _ in range(3):
                 graph.replay()
             torch.cuda.synchronize(self.device)
@@ -158,10 +159,21 @@ class ModelRunner:
             for _ in range(10):
                 graph.replay()
             torch.cuda.synchronize(self.device)
-            seconds.append(time.perf_counter() - start)
-            del self.graphs[bucket], graph
-        best = min(range(len(choices)), key=lambda i: seconds[i])
-        ops.keep_large_weight_rows(choices[best] if seconds[best] < 0.97 * seconds[0] else choices[0])
+            return time.perf_counter() - start
+
+        kept = self._capture(bucket)
+        choices = offers()
+        if len(choices) < 2:
+            return
+        best, best_seconds = choices[0], 0.97 * seconds(kept[0])
+        for rows in choices[1:]:
+            ops.try_large_weight_rows(rows)
+            trial = self._capture(bucket)
+            took = seconds(trial[0])
+            if took < best_seconds:
+                best, best_seconds, kept = rows, took, trial
+        ops.keep_large_weight_rows(best)
+        self.graphs[bucket] = kept
 
     def dummy_step(self, num_tokens: int, num_entries: int) -> int:
         """Run one step of `num_tokens` zero tokens in `num_entries` requests (fewer of
