@@ -566,6 +566,12 @@ def test_attend_in_a_large_decode_step(ops, gpu_device, window):
     assert ops._decode_splits(8 * 3 * len(DECODE_SPANS), 1024) == 1
     attend_decode_case(ops, gpu_device, torch.bfloat16, 16, 8, 128, 16, window, DECODE_SPANS * 3)
     attend_decode_case(ops, gpu_device, torch.bfloat16, 16, 8, 128, 16, window, DECODE_SPANS * 7)
+    # and so many that the kernel for long portions takes the single tokens as its items
+    many = DECODE_SPANS * 13
+    batch, _, _, _ = paged_scenario(gpu_device, torch.bfloat16, nkv=8, hd=128, page_size=16,
+                                    spans=many, seed=51, fill=False)
+    assert ops._prefill_tiles(batch, 8, 2) is not None
+    attend_decode_case(ops, gpu_device, torch.bfloat16, 16, 8, 128, 16, window, many)
 
 
 def attend_decode_case(ops, gpu_device, dtype, nq, nkv, hd, page, window, spans):

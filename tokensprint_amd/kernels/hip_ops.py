@@ -793,8 +793,12 @@ class HipOps:
         tokens_per_tile = 16 // min(group, 16)
         tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
         waves = tiles16 * num_kv_heads * -(-group // 16)
-        # a step of single tokens only takes it where the chip is full without splitting keys
-        enough = 256 if batch.max_q_len >= 32 else 2048
+        # a step of single tokens only takes it where the chip is full without splitting keys:
+        # from 1,024 wave tiles (128 entries at 8 key/value heads) it is ahead of the general
+        # kernel at every context length tried (136 entries: 34 against 41 us at 300 tokens
+        # each, 130 against 150 at 100 to 2,000, 426 against 445 at 4,000; 200 entries: 46
+        # / 51, 180 / 223, 608 / 653), at 576 to 768 it is level or behind
+        enough = 256 if batch.max_q_len >= 32 else 1024
         return tokens_per_tile if waves >= enough else None
 
     def _attention_tiles(self, batch, tokens, longest_first=False):
