@@ -318,6 +318,13 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b * args.steps / d, 1)
             del e
             torch.cuda.empty_cache()
+        # more requests than the captured decode kernels for few rows take (the library's
+        # products and norm kernels from 65 rows on): 128 tokens decoded behind the same prompts
+        _, e = make_engine(raw, args.dtype, layers, 256, ctx_len, 8192, page, model=model)
+        d, _ = decode_run(e, 256, args.prompt_len, 112, 16, vocab)
+        points["decode_b256"] = round(256 * 112 / d, 1)
+        del e
+        torch.cuda.empty_cache()
         # longer contexts: 128 tokens decoded behind prompts that end 256 short of the length
         for b in (8, 64):
             for ctx in (2048, 4096):
