@@ -3,9 +3,12 @@
     python bench.py --gpus 1 --steps K --warmup W
 
 A step is one decode step of the engine (schedule, run, sample, postprocess) for a batch
-of 8 requests with 512-token prompts; `value` is decoded tokens per second.  The same
-line carries a 2,048-token prefill, decode at batch 1 and 64, and the decode step's
-fraction of the HBM roofline.  Peaks are MI355X's published ones.
+of 8 requests with 512-token prompts; `value` is decoded tokens per second, counted from
+the tokens the requests received in the timed steps.  The same line carries a 2,048-token
+prefill, decode at batch 1, 64 and 256 and at longer contexts (`points`, with each
+point's fraction of the HBM rate, mean context and step time beside it), the split of a
+step into products and attention, a float32 decode point, and the decode step's fraction
+of the HBM roofline.  Peaks are MI355X's published ones.
 """
 
 from __future__ import annotations
@@ -38,32 +41,75 @@ def make_engine(raw, dtype, layers, batch, max_len, budget, page_size, seed=0, m
     return model, LLMEngine(model, config)
 
 
-def decode_run(engine, batch, prompt_len, steps, warmup, vocab):
-    """Prefill `batch` prompts, then time exactly `steps` decode steps."""
+def decode_points(batch, prompt_len, steps, warmup, context=4096):
+    """Every decode measurement of a run: name -> (requests, prompt tokens, timed steps,
+    warm-up steps, token budget of a step).  The first is the headline.  The same prompts
+    and number of decoded tokens at batch 1 and 64; more requests than the captured decode
+    kernels for few rows take (the library's products and norm kernels from 65 rows on) at
+    256; and contexts of 2,048 and 4,096 tokens, reached by prompts that end 256 short of
+    them."""
+    points = {"headline": (batch, prompt_len, steps, warmup, 2048)}
+    for b in (1, 64):
+        points[f"decode_b{b}"] = (b, prompt_len, steps, warmup, 2048)
+    points["decode_b256"] = (256, prompt_len, min(steps, 112), min(warmup, 16), 8192)
+    for b in (8, 64):
+        for ctx in (context // 2, context):
+            points[f"decode_b{b}_ctx{ctx}"] = (b, ctx - 256, min(steps, 112), min(warmup, 16),
+                                               8192)
+    return points
+
+
+def decode_lengths(batch, prompt_len, steps, warmup, budget):
+    """(max_model_len, max_tokens) with which `decode_run` keeps every request alive to the
+    end of the timed steps.  A request whose prompt is through decodes beside the others'
+    prompt portions, one token a step, so the first one is ahead of the last by the
+    number of steps the prompts take; nobody may reach a limit before the last timed step."""
+    prefill_steps = -(-batch * prompt_len // budget) + batch
+    max_tokens = prefill_steps + warmup + steps + 8
+    return prompt_len + max_tokens + 1, max_tokens
+
+
+def decode_run(engine, batch, prompt_len, steps, warmup, vocab, max_tokens):
+    """Prefill `batch` prompts, then time exactly `steps` decode steps.  Returns (seconds,
+    tokens decoded in them, mean over the timed steps of the tokens all live requests
+    hold).  The decoded tokens are counted from the requests, and every request must be
+    live and decoding from the first timed step to the last."""
     import torch
     from tokensprint_amd.config import SamplingParams
     g = torch.Generator().manual_seed(0)
-    params = SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True)
+    params = SamplingParams(temperature=0.0, max_tokens=max_tokens, ignore_eos=True)
     for _ in range(batch):
         engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(), params)
-    while any(r.num_completion_tokens == 0 for r in engine.requests.values()):
+    reqs = list(engine.requests.values())
+    while any(r.num_completion_tokens == 0 for r in reqs):
         engine.step()                      # prefill portions until every request has a token
     for _ in range(warmup):
         engine.step()
-    ctx0 = sum(len(r) for r in engine.requests.values())
-    torch.cuda.synchronize()
+    sync = torch.cuda.synchronize if torch.cuda.is_available() else (lambda: None)
+    live0 = len(engine.scheduler.running)
+    done0 = sum(r.num_completion_tokens for r in reqs)
+    ctx0 = sum(len(r) for r in engine.scheduler.running)
+    sync()
     t0 = time.perf_counter()
     for _ in range(steps):
         engine.step()
-    torch.cuda.synchronize()
+    sync()
     dt = time.perf_counter() - t0
-    ctx1 = sum(len(r) for r in engine.requests.values())
-    # drop the requests
+    live1 = len(engine.scheduler.running)
+    decoded = sum(r.num_completion_tokens for r in reqs) - done0
+    ctx1 = sum(len(r) for r in engine.scheduler.running)
+    if live0 != batch or live1 != batch or decoded != batch * steps:
+        raise RuntimeError(
+            f"decode run of {batch} requests: {live0} live before and {live1} after the timed "
+            f"steps, {decoded} tokens decoded where {batch * steps} were expected")
+    # drop the requests (one step may still be in flight: let it land first)
+    sync()
+    engine._flight = None
     for r in list(engine.scheduler.running):
         engine.scheduler.manager.free(r.cache)
     engine.scheduler.running.clear()
     engine.requests.clear()
-    return dt, (ctx0 + ctx1) / 2.0
+    return dt, decoded, (ctx0 + ctx1) / 2.0
 
 
 PRODUCTS = ("linear", "norm_linear", "linear_into_stream", "linear_silu_mul")
@@ -207,6 +253,18 @@ def prefill_run(engine, tokens, vocab, reps=5):
     return times[len(times) // 2]
 
 
+def cache_bytes(model, context, item) -> float:
+    """Bytes of cache a decode step reads for one request that holds `context` tokens: of
+    every run that owns a paged cache, keys and values of the tokens its mixer can see
+    (all of them, or a window's)."""
+    total = 0.0
+    for need in model.cache_needs():
+        if need is not None and hasattr(need, "num_kv_heads"):
+            seen = context if need.window is None else min(context, need.window)
+            total += 2 * need.num_kv_heads * need.head_dim * item * seen
+    return total
+
+
 def prefill_attention_flops(cfg, T) -> float:
     """Causal QK^T and PV of one layer for one prompt of T tokens."""
     return 2 * 2 * cfg["num_attention_heads"] * cfg["head_dim"] * T * (T + 1) / 2
@@ -230,6 +288,7 @@ def main() -> int:
     ap.add_argument("--model", default="qwen3-0.6b")
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode run")
+    ap.add_argument("--skip-fp32", action="store_true", help="no float32 decode point")
     ap.add_argument("--only-prefill", action="store_true",
                     help="only the 2,048-token prefill (for profiling); prints its own line")
     args = ap.parse_args()
@@ -254,22 +313,30 @@ def main() -> int:
         print(json.dumps({"prefill_ms": round(sec * 1e3, 3), "tokens": 2048,
                           "tok_per_s": round(2048 / sec, 1)}))
         return 0
-    model, engine = make_engine(raw, args.dtype, layers, args.batch, ctx_len, 2048, page)
-    wbytes = model.step_weight_bytes()   # every weight a decode step reads, each once
-    kv_per_token = 2 * layers * raw["num_key_value_heads"] * raw["head_dim"] * item
+    plan = decode_points(args.batch, args.prompt_len, args.steps, args.warmup, ctx_len)
+    if args.skip_points:
+        plan = {"headline": plan["headline"]}
+    model, results = None, {}
+    for name, (b, prompt_len, steps, warmup, budget) in plan.items():
+        max_len, max_tokens = decode_lengths(b, prompt_len, steps, warmup, budget)
+        model, engine = make_engine(raw, args.dtype, layers, b, max_len, budget, page,
+                                    model=model)
+        if name == "headline":
+            wbytes = model.step_weight_bytes()   # every weight a decode step reads, each once
+        sec, decoded, held = decode_run(engine, b, prompt_len, steps, warmup, vocab, max_tokens)
+        step_bytes = wbytes + cache_bytes(model, held / b, item) * b
+        results[name] = {"tok_s": decoded / sec, "ms_step": sec / steps * 1e3,
+                         "context": held / b, "gbs": step_bytes * steps / sec / 1e9}
+        del engine
+        torch.cuda.empty_cache()
 
-    dt, mean_tokens = decode_run(engine, args.batch, args.prompt_len, args.steps, args.warmup,
-                                 vocab)
-    ms_step = dt / args.steps * 1e3
-    value = args.batch * args.steps / dt
-    step_bytes = wbytes + kv_per_token * mean_tokens
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
-
+    head = results["headline"]
     out = {
         "metric": f"decode tok/s at batch {args.batch} ({args.model} shape, "
                   f"{args.prompt_len}-token prompts)",
-        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "value": round(head["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(head["ms_step"], 4),
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dt_name,
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02) seed 0",
         "config": {
@@ -279,23 +346,25 @@ def main() -> int:
             "num_kv_heads": raw["num_key_value_heads"], "head_dim": raw["head_dim"],
             "intermediate_size": raw["intermediate_size"], "vocab_size": vocab,
             "tied_embeddings": raw["tie_word_embeddings"], "prompt_len": args.prompt_len,
-            "page_size": page, "mean_context": round(mean_tokens / args.batch, 1),
+            "page_size": page, "mean_context": round(head["context"], 1),
         },
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4)},
     }
 
     if not args.skip_points:
         # where the decode step's time goes, from captured steps with one kind of kernel
         # taken out: products against the weights they stream, attention against the cache
-        context = int(round(mean_tokens / args.batch))
-        whole, t_products, t_attention = step_split(model, page, decode_entries(args.batch, context),
-                                                    ctx_len)
-        out["roofline"]["products_gbs"] = round(wbytes / t_products / 1e9, 1)
-        out["roofline"]["products_us"] = round(t_products * 1e6, 1)
-        out["roofline"]["attention_gbs"] = round(kv_per_token * args.batch * context / t_attention / 1e9, 1)
-        out["roofline"]["attention_us"] = round(t_attention * 1e6, 1)
-        out["roofline"]["step_us_without_host"] = round(whole * 1e6, 1)
+        def split(b, context, into, prefix=""):
+            whole, t_products, t_attention = step_split(model, page, decode_entries(b, context),
+                                                        ctx_len)
+            into[prefix + "products_gbs"] = round(wbytes / t_products / 1e9, 1)
+            into[prefix + "products_us"] = round(t_products * 1e6, 1)
+            into[prefix + "attention_gbs"] = round(
+                cache_bytes(model, context, item) * b / t_attention / 1e9, 1)
+            into[prefix + "attention_us"] = round(t_attention * 1e6, 1)
+            into[prefix + "step_us_without_host"] = round(whole * 1e6, 1)
+        split(args.batch, int(round(head["context"])), out["roofline"])
 
         T = 2048
         _, pre_engine = make_engine(raw, args.dtype, layers, 1, ctx_len, T, page, model=model)
@@ -311,29 +380,33 @@ def main() -> int:
         out["prefill"]["attention_tflops"] = round(attn_flops / t_attention / 1e12, 1)
         out["prefill"]["attention_us"] = round(t_attention * 1e6, 1)
         del pre_engine
-        points = {}
-        for b in (1, 64):       # the same prompts and number of decoded tokens as the headline run
-            _, e = make_engine(raw, args.dtype, layers, b, ctx_len, 2048, page, model=model)
-            d, _ = decode_run(e, b, args.prompt_len, args.steps, args.warmup, vocab)
-            points[f"decode_b{b}"] = round(b * args.steps / d, 1)
-            del e
-            torch.cuda.empty_cache()
-        # more requests than the captured decode kernels for few rows take (the library's
-        # products and norm kernels from 65 rows on): 128 tokens decoded behind the same prompts
-        _, e = make_engine(raw, args.dtype, layers, 256, ctx_len, 8192, page, model=model)
-        d, _ = decode_run(e, 256, args.prompt_len, 112, 16, vocab)
-        points["decode_b256"] = round(256 * 112 / d, 1)
-        del e
         torch.cuda.empty_cache()
-        # longer contexts: 128 tokens decoded behind prompts that end 256 short of the length
-        for b in (8, 64):
-            for ctx in (2048, 4096):
-                _, e = make_engine(raw, args.dtype, layers, b, ctx_len, 2048, page, model=model)
-                d, _ = decode_run(e, b, ctx - 256, 112, 16, vocab)
-                points[f"decode_b{b}_ctx{ctx}"] = round(b * 112 / d, 1)
-                del e
-                torch.cuda.empty_cache()
-        out["points"] = points
+        names = [n for n in results if n != "headline"]
+        out["points"] = {n: round(results[n]["tok_s"], 1) for n in names}
+        # of every point: its fraction of the HBM rate (weights once and the live requests'
+        # cache, over its measured step), the mean context it was measured at, its step
+        out["points_frac"] = {n: round(results[n]["gbs"] / HBM_PEAK_GBS, 4) for n in names}
+        out["points_context"] = {n: round(results[n]["context"], 1) for n in names}
+        out["points_ms_per_step"] = {n: round(results[n]["ms_step"], 4) for n in names}
+        out["points_split"] = {}
+        for n in ("decode_b1", "decode_b64"):
+            split(plan[n][0], int(round(results[n]["context"])), out["points_split"], n + "_")
+        if dt_name == "bf16" and not args.skip_fp32:
+            # the true 32-bit path at the headline's batch: its own weights, cache and kernels
+            del model
+            torch.cuda.empty_cache()
+            b, prompt_len, steps, warmup, budget = plan["headline"]
+            steps, warmup = min(steps, 48), min(warmup, 4)
+            max_len, max_tokens = decode_lengths(b, prompt_len, steps, warmup, budget)
+            model32, engine = make_engine(raw, "float32", layers, b, max_len, budget, page)
+            sec, decoded, held = decode_run(engine, b, prompt_len, steps, warmup, vocab,
+                                            max_tokens)
+            bytes32 = model32.step_weight_bytes() + cache_bytes(model32, held / b, 4) * b
+            out["points"][f"decode_b{b}_fp32"] = round(decoded / sec, 1)
+            out["points_frac"][f"decode_b{b}_fp32"] = round(
+                bytes32 * steps / sec / 1e9 / HBM_PEAK_GBS, 4)
+            out["points_context"][f"decode_b{b}_fp32"] = round(held / b, 1)
+            out["points_ms_per_step"][f"decode_b{b}_fp32"] = round(sec / steps * 1e3, 4)
     print(json.dumps(out))
     return 0
 
