@@ -3,12 +3,14 @@ synthetic workload of token-id prompts with random prompt and output lengths, on
 warm-up request, then output tokens divided by wall time with a device synchronisation
 on both sides.  Options keep the reference's names and meanings (booleans take a value:
 `--use-tqdm False`); the comparison backend of the reference is not part of this engine.
-Weights are random unless --model-dir names a checkpoint folder.
+Weights are random (of --model-name's configuration, or of the config.json that
+--config-json names) unless --model-dir names a checkpoint folder.
 """
 
 from __future__ import annotations
 
 import argparse
+import json
 import tempfile
 import time
 from pathlib import Path
@@ -28,6 +30,8 @@ def parse_args(argv=None):
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model-name", default="qwen/qwen3-0.6b")
     ap.add_argument("--model-dir", type=Path, default=None)
+    ap.add_argument("--config-json", type=Path, default=None,
+                    help="random weights of this config.json instead of --model-name's")
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--max-input-len", type=int, default=1024)
     ap.add_argument("--max-output-len", type=int, default=1024)
@@ -76,7 +80,8 @@ def main(args) -> None:
         _, model = load_model(args.model_dir, args.dtype, "cuda:0")
         model_dir = str(args.model_dir)
     else:
-        raw = load_named_config(args.model_name)
+        raw = json.loads(args.config_json.read_text()) if args.config_json is not None \
+            else load_named_config(args.model_name)
         if args.layers:
             raw["num_hidden_layers"] = args.layers
         _, model = random_model(raw, 0, args.dtype, "cuda:0")

@@ -3,8 +3,9 @@
 Same options with the same meanings (--model-name, --cache-dir, --prompt, --max-tokens,
 --temperature, --enforce-eager; booleans take a value, `--enforce-eager True`, as the
 reference's FlagConversionOff does), plus what an engine without network needs:
---model-dir, --dtype, --random-weights SEED, --prompt-ids, and the cache and scheduler
-knobs of the engine configuration.
+--model-dir, --dtype, --random-weights SEED (for --model-name, or for the config.json that
+--config-json names), --prompt-ids, and the cache and scheduler knobs of the engine
+configuration.
 """
 
 from __future__ import annotations
@@ -43,6 +44,8 @@ def parse_args(argv=None):
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
                     help="write a random-weights folder for --model-name and run that")
+    ap.add_argument("--config-json", type=Path, default=None,
+                    help="with --random-weights: this config.json instead of --model-name's")
     ap.add_argument("--prompt-ids", default=None,
                     help="comma-separated token ids instead of --prompt (no tokenizer needed)")
     ap.add_argument("--page-size", type=int, default=16)
@@ -73,8 +76,11 @@ def main(args) -> None:
     model_dir = args.model_dir
     if args.random_weights is not None:
         model_dir = model_dir or Path(tempfile.mkdtemp(prefix="tokensprint_random_"))
-        write_random_model(model_dir, load_named_config(args.model_name), args.random_weights,
-                           dtype)
+        raw = json.loads(args.config_json.read_text()) if args.config_json is not None \
+            else load_named_config(args.model_name)
+        write_random_model(model_dir, raw, args.random_weights, dtype)
+    elif args.config_json is not None:
+        raise ValueError("--config-json describes random weights: give --random-weights SEED")
     elif model_dir is None:
         model_dir = args.cache_dir / get_model_repo_id(args.model_name).split("/")[-1]
     _, model = load_model(model_dir, dtype, "cuda:0")

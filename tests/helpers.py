@@ -57,3 +57,30 @@ GPU_ONLY = {"E": (LAYER_E, 4, 16), "F": (LAYER_F, 5, 16), "G": (LAYER_G, 6, 16)}
 def random_prompt(length, vocab, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (length,), generator=g).tolist()
+
+
+def write_word_tokenizer(model_dir, vocab_size, *, eos_id=2, name_eos=True, pad_id=None):
+    """A word-level tokenizer for `vocab_size` ids in `model_dir`, as checkpoint folders
+    hold one: tokenizer.json (word i is "w<i>", split at white space; id 0 is the unknown
+    word, `eos_id` the end-of-sequence token, both special) and tokenizer_config.json."""
+    import json
+    from pathlib import Path
+
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    words = {f"w{i}": i for i in range(vocab_size)}
+    words = {("<unk>" if i == 0 else "<eos>" if i == eos_id else "<pad>" if i == pad_id else w): i
+             for w, i in words.items()}
+    tok = Tokenizer(models.WordLevel(words, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.add_special_tokens(["<unk>", "<eos>"] + (["<pad>"] if pad_id is not None else []))
+    model_dir = Path(model_dir)
+    model_dir.mkdir(parents=True, exist_ok=True)
+    tok.save(str(model_dir / "tokenizer.json"))
+    named = {"unk_token": "<unk>"}
+    if name_eos:
+        named["eos_token"] = {"content": "<eos>", "special": True}
+    if pad_id is not None:
+        named["pad_token"] = "<pad>"
+    (model_dir / "tokenizer_config.json").write_text(json.dumps(named))
+    return tok

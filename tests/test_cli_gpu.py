@@ -12,11 +12,17 @@ from pathlib import Path
 import pytest
 import torch
 
-from helpers import random_prompt
+from helpers import TINY_A, TINY_B, random_prompt, write_word_tokenizer
 from plain import qwen3_plain as plain
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
+
+
+def config_json(tmp_path, cfg):
+    path = tmp_path / "config_for_random_weights.json"
+    path.write_text(json.dumps(cfg))
+    return path
 
 
 def run_program(args, timeout=300):
@@ -35,7 +41,8 @@ def run_program(args, timeout=300):
 def test_run_py_generates_the_plain_tokens(gpu_device, tmp_path, dtype, extra):
     prompt = random_prompt(19, 389, 5)
     model_dir = tmp_path / "tiny-b"
-    proc = run_program(["run.py", "--model-name", "tiny-b", "--random-weights", "1",
+    proc = run_program(["run.py", "--config-json", config_json(tmp_path, TINY_B),
+                        "--random-weights", "1",
                         "--model-dir", model_dir, "--dtype", dtype, "--temperature", "0",
                         "--max-tokens", "14", "--ignore-eos", "True", "--max-num-seqs", "16",
                         "--prompt-ids", ",".join(map(str, prompt)), *extra])
@@ -52,7 +59,8 @@ def test_run_py_bfloat16_runs_and_samples(gpu_device, tmp_path):
     prompt = random_prompt(40, 256, 6)
     out = []
     for _ in range(2):
-        proc = run_program(["run.py", "--model-name", "tiny/tiny-a", "--random-weights", "0",
+        proc = run_program(["run.py", "--config-json", config_json(tmp_path, TINY_A),
+                            "--random-weights", "0",
                             "--model-dir", tmp_path / "tiny-a", "--temperature", "0.8",
                             "--max-tokens", "9", "--ignore-eos", "True", "--max-num-seqs", "8",
                             "--page-size", "4", "--seed", "11",
@@ -62,8 +70,36 @@ def test_run_py_bfloat16_runs_and_samples(gpu_device, tmp_path):
     assert out[0] == out[1]                         # a seeded draw: the same tokens again
 
 
-def test_benchmark_py(gpu_device):
-    proc = run_program(["benchmark.py", "--model-name", "tiny-b", "--num-seqs", "8",
+def test_run_py_with_a_text_prompt(gpu_device, tmp_path):
+    """The text path (run.py:42-68 of the reference): the folder's tokenizer encodes the
+    prompt, its end-of-sequence token ends the request, and what is printed is its
+    decoding of the completion without special tokens."""
+    from tokensprint_amd.weights import write_random_model
+    model_dir = tmp_path / "tiny-b-with-tokenizer"
+    write_random_model(model_dir, TINY_B, 1, torch.float32)
+    pcfg, w = plain.read_model_dir(model_dir)
+    prompt = [t or 1 for t in random_prompt(19, 389, 5)]          # id 0 is the unknown word
+    completion = plain.greedy_generate(pcfg, w, prompt, 14)
+    # the end-of-sequence token: one the greedy completion meets for the first time after
+    # a few tokens, so that the request has to stop there
+    stop = next(k for k in range(3, 14) if completion[k] not in completion[:k] + [0])
+    eos = completion[stop]
+    tok = write_word_tokenizer(model_dir, TINY_B["vocab_size"], eos_id=eos)
+    text = " ".join(tok.id_to_token(t) for t in prompt)
+    assert tok.encode(text).ids == prompt
+    common = ["run.py", "--model-dir", model_dir, "--dtype", "float32", "--temperature", "0",
+              "--max-tokens", "14", "--max-num-seqs", "16", "--prompt", text]
+    proc = run_program(common)
+    assert proc.stdout.strip().splitlines()[-1] == tok.decode(completion[:stop])
+    assert f"EOS {eos}" in proc.stderr and "TextTokenizer" in proc.stderr
+    proc = run_program(common + ["--ignore-eos", "True"])
+    assert proc.stdout.strip().splitlines()[-1] == tok.decode(completion)   # skips the special one
+    assert len(tok.decode(completion).split()) == sum(t not in (0, eos) for t in completion)
+
+
+def test_benchmark_py(gpu_device, tmp_path):
+    proc = run_program(["benchmark.py", "--config-json", config_json(tmp_path, TINY_B),
+                        "--num-seqs", "8",
                         "--max-input-len", "120", "--max-output-len", "120",
                         "--max-num-seqs", "8", "--use-tqdm", "False"])
     line = [ln for ln in proc.stdout.splitlines() if "Throughput" in ln][-1]
@@ -71,8 +107,9 @@ def test_benchmark_py(gpu_device):
     assert m and int(m.group(1)) >= 8 * 100 and float(m.group(3)) > 0, line
 
 
-def test_benchmark_py_with_a_pool_that_forces_preemption(gpu_device):
-    proc = run_program(["benchmark.py", "--model-name", "tiny-b", "--num-seqs", "6",
+def test_benchmark_py_with_a_pool_that_forces_preemption(gpu_device, tmp_path):
+    proc = run_program(["benchmark.py", "--config-json", config_json(tmp_path, TINY_B),
+                        "--num-seqs", "6",
                         "--min-input-len", "100", "--max-input-len", "100",
                         "--min-output-len", "60", "--max-output-len", "60",
                         "--max-num-seqs", "6", "--num-pages", "30", "--use-tqdm", "False",
@@ -84,5 +121,5 @@ def test_benchmark_py_with_a_pool_that_forces_preemption(gpu_device):
 def test_model_registry_py():
     proc = run_program(["model_registry.py"])
     assert "qwen:\n  - qwen3-0.6b (qwen/qwen3-0.6b)" in proc.stdout
-    assert "  - tiny-b (tiny/tiny-b)" in proc.stdout
+    assert "tiny" not in proc.stdout               # test configurations are no presets
     assert "Qwen3ForCausalLM" in proc.stdout

@@ -107,8 +107,21 @@ def test_named_0_6b_matches_the_reference_factory():
                                        1_000_000.0, 1e-6, True)
 
 
-def test_tiny_presets_are_the_tiny_test_configurations():
-    from helpers import TINY_A, TINY_B
-    assert resolve_model_name("tiny/tiny-b") == "tiny-b" and not model_is_registered("qwen/tiny-a")
-    for name, cfg in (("tiny-a", TINY_A), ("tiny-b", TINY_B)):
-        assert Qwen3Config.from_dict(load_named_config(name)) == Qwen3Config.from_dict(cfg)
+def test_a_model_registered_by_name_at_run_time(tmp_path):
+    # what a user (or a test) adds with register_named_model is found by short and long
+    # name like the shipped presets; a short name is unique over all families
+    import json
+    from helpers import TINY_B
+    from tokensprint_amd.config.registry import _NAMED, register_named_model
+    preset = tmp_path / "tiny-b.json"
+    preset.write_text(json.dumps(TINY_B))
+    register_named_model("tiny", "tiny-b", preset)
+    try:
+        assert resolve_model_name("tiny/tiny-b") == "tiny-b"
+        assert not model_is_registered("qwen/tiny-b")
+        assert Qwen3Config.from_dict(load_named_config("tiny-b")) == Qwen3Config.from_dict(TINY_B)
+        with pytest.raises(ValueError, match="already registered"):
+            register_named_model("qwen", "tiny-b", preset)
+    finally:
+        _NAMED.pop("tiny-b")
+    assert not model_is_registered("tiny-b")      # the shipped presets hold real models only
