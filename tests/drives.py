@@ -15,12 +15,16 @@ from tokensprint_amd.engine import StepEntry
 class Collector:
     def __init__(self):
         self.rows = {}     # request id -> {position: logits row}
+        self.earlier = []  # (request id, position, row) computed before and computed again since
 
     def take(self, entries, logits):
         r = 0
         for e in entries:
             for w in e.want:
-                self.rows.setdefault(e.cache.request_id, {})[e.start + w] = logits[r].cpu()
+                got = self.rows.setdefault(e.cache.request_id, {})
+                if e.start + w in got:
+                    self.earlier.append((e.cache.request_id, e.start + w, got[e.start + w]))
+                got[e.start + w] = logits[r].cpu()
                 r += 1
         assert r == logits.shape[0]
 
@@ -123,6 +127,53 @@ def drive_mixed(runner, requests, max_live=4, seed=0, decode_tail=12):
     return col
 
 
+def drive_preempted(runner, requests, max_live=4, seed=0, decode_tail=12, every=5):
+    """The mixed drive, with requests taken out mid-way as a scheduler does that runs out
+    of pages: every `every`-th step a live request that has come some way gives back all
+    it holds and starts again from its first token, in portions, beside the others'
+    portions and decoded tokens.  Logits are collected on both passes."""
+    g = torch.Generator().manual_seed(seed)
+    col = Collector()
+    waiting = list(requests.items())
+    live = {}       # rid -> [rc, tokens, pos, times preempted]
+    preemptions = {rid: 0 for rid in requests}
+    steps = 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, tokens = waiting.pop(0)
+            live[rid] = [runner.manager.admit(rid), tokens, 0]
+        steps += 1
+        assert steps < 10000, "preempting drive makes no progress"
+        if steps % every == 0:
+            victims = [rid for rid, st in live.items() if st[2] >= 3 and preemptions[rid] < 2]
+            if victims:
+                rid = victims[int(torch.randint(0, len(victims), (1,), generator=g))]
+                runner.manager.free(live[rid][0])
+                live[rid] = [runner.manager.admit(rid), live[rid][1], 0]
+                preemptions[rid] += 1
+        entries, ended = [], []
+        for rid, state in live.items():
+            rc, tokens, pos = state
+            remaining = len(tokens) - pos
+            n = 1 if remaining <= decode_tail else \
+                min(int(torch.randint(2, 24, (1,), generator=g)), remaining - decode_tail)
+            if not runner.manager.can_extend(rc, pos + n):
+                continue
+            runner.manager.extend(rc, pos + n)
+            entries.append(StepEntry(rc, tokens[pos:pos + n], pos, list(range(n))))
+            state[2] = pos + n
+            if state[2] == len(tokens):
+                ended.append(rid)
+        if not entries:
+            continue
+        col.take(entries, runner.step(entries))
+        for rid in ended:
+            runner.manager.free(live.pop(rid)[0])
+        runner.manager.check()
+    assert sum(preemptions.values()) >= 2 and col.earlier
+    return col
+
+
 def row_tolerance(ref, rtol, atol):
     """Allowed |got - ref| per element.  `atol` is in units of the request's largest
     logit, never less than one: a product's rounding error grows with the magnitudes it
@@ -147,3 +198,10 @@ def compare(col, plain_logits, rtol, atol):
                 f"request {rid}: first wrong position {p} of {ref.shape[0]}, "
                 f"max abs error there {err:.3e}, overall {(got - ref).abs().max():.3e}, "
                 f"largest logit {float(ref.abs().max()):.3f}")
+    # rows that were computed once more later (after a preemption): the first pass too
+    for rid, p, row in col.earlier:
+        ref = plain_logits[rid]
+        err = (row - ref[p]).abs()
+        if not bool((err <= row_tolerance(ref, rtol, atol)[p]).all()):
+            raise AssertionError(f"request {rid}: position {p} was wrong before its request "
+                                 f"was preempted, max abs error {err.max():.3e}")

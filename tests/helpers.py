@@ -52,6 +52,12 @@ LAYER_F = qwen3_config(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128
 LAYER_G = qwen3_config(hidden=5120, layers=2, heads=64, kv_heads=8, head_dim=128, inter=25600,
                        vocab=20011, eps=1e-6, theta=1e6, tied=False, max_pos=256)
 GPU_ONLY = {"E": (LAYER_E, 4, 16), "F": (LAYER_F, 5, 16), "G": (LAYER_G, 6, 16)}
+# The same widths with a windowed layer beside a full one: two cache groups, so that a
+# step (a captured decode step too) carries two block tables and the window's kernels run
+# at the widths of real models.
+WINDOWED = {name + "W": (dict(cfg, sliding_window=40, use_sliding_window=True,
+                              layer_types=["sliding_attention", "full_attention"]), seed + 10, page)
+            for name, (cfg, seed, page) in GPU_ONLY.items()}
 
 
 def random_prompt(length, vocab, seed):

@@ -56,3 +56,10 @@ def test_mixed_with_page_reuse(setup):
     runner = runner_for(model, page, 160 // page)
     drives.compare(drives.drive_mixed(runner, requests), ref, 1e-4, 2e-5)
     assert all(pool.num_used == 0 for pool in runner.manager.pools)
+
+
+def test_preempted_and_recomputed(setup):
+    model, page, requests, ref = setup
+    runner = runner_for(model, page, 160 // page)
+    drives.compare(drives.drive_preempted(runner, requests), ref, 1e-4, 2e-5)
+    assert all(pool.num_used == 0 for pool in runner.manager.pools)

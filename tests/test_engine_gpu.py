@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import drives
-from helpers import GPU_ONLY, TINY, random_prompt
+from helpers import GPU_ONLY, TINY, WINDOWED, random_prompt
 from plain import qwen3_plain as plain
 from tokensprint_amd.engine import ModelRunner
 from tokensprint_amd.engine.assemble import load_model
@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 TOL = {torch.float32: (1e-4, 2e-5), torch.bfloat16: (3e-2, 3e-2)}
 
 
-CONFIGS = {**TINY, **GPU_ONLY}
+CONFIGS = {**TINY, **GPU_ONLY, **WINDOWED}
 
 
 @pytest.fixture(scope="module", params=[(n, d) for n in sorted(CONFIGS)
@@ -29,7 +29,9 @@ def setup(request, tmp_path_factory, gpu_device):
     name, dtype = request.param
     cfg, seed, page = CONFIGS[name]
     d = tmp_path_factory.mktemp(f"tiny{name}")
-    write_random_model(d, cfg, seed, dtype)
+    # (the wide models' values are drawn on the GPU, which takes a second where the CPU
+    # takes a minute)
+    write_random_model(d, cfg, seed, dtype, device="cpu" if name in TINY else gpu_device)
     pcfg, w = plain.read_model_dir(d)          # the same (rounded) weights, held in float32
     _, model = load_model(d, dtype, gpu_device)
     lengths = [5, 11, 17, 40, 64, 1, 23, 100]
@@ -65,6 +67,17 @@ def test_mixed_with_page_reuse(setup):
     model, page, requests, ref, (rtol, atol) = setup
     runner = runner_for(model, page, 224 // page)      # 261 tokens in all: pages are reused
     drives.compare(drives.drive_mixed(runner, requests), ref, rtol, atol)
+    assert all(pool.num_used == 0 for pool in runner.manager.pools)
+
+
+def test_preempted_and_recomputed(setup):
+    """Requests that give everything back mid-way and are computed again from their first
+    token beside the others' portions and decoded tokens (what the scheduler does when
+    pages run out, engine/generation/scheduler.py:95-108,177-180 of the reference): the
+    logits of both passes."""
+    model, page, requests, ref, (rtol, atol) = setup
+    runner = runner_for(model, page, 224 // page)
+    drives.compare(drives.drive_preempted(runner, requests), ref, rtol, atol)
     assert all(pool.num_used == 0 for pool in runner.manager.pools)
 
 

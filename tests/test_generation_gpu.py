@@ -81,6 +81,7 @@ def test_prefix_cache_gives_the_same_tokens(setup):
         assert engine.generate(shared, sp, use_tqdm=False) == want, blocks
         assert engine.generate(shared[::-1], sp, use_tqdm=False) == want[::-1], blocks
         assert engine.scheduler.num_prefix_hit_tokens >= 3 * page
+        assert engine.num_steps_ahead > 0           # decode steps were launched ahead meanwhile
         engine.runner.manager.check()
         assert all(p.num_used == 0 for p in engine.runner.manager.pools)
 
@@ -248,3 +249,50 @@ def test_warm_up_chooses_who_multiplies_large_weights(setup, gpu_device, tmp_pat
                 pos += n
             runner.manager.free(rc)
         assert runner.graphs
+
+
+def assert_near_greedy(pcfg, w, prompt, completion, rtol, atol):
+    """A greedy completion from reduced-precision logits, checked at the logit level: at
+    every position the token that was drawn has a plain logit within two tolerances of the
+    plain maximum there (the engine's own logits of the drawn token and of the plain
+    argmax are each within one tolerance of the plain ones)."""
+    import drives
+    ref = plain.forward_logits(pcfg, w, prompt + completion[:-1])
+    for i, token in enumerate(completion):
+        row = ref[len(prompt) - 1 + i]
+        slack = 2 * drives.row_tolerance(ref, rtol, atol)[len(prompt) - 1 + i]
+        best = int(row.argmax())
+        assert row[token] >= row[best] - max(slack[token], slack[best]), \
+            f"token {i}: drew {token} ({row[token]:.4f}), plain argmax {best} ({row[best]:.4f})"
+
+
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_bfloat16_with_prefix_cache_steps_ahead_and_preemption(name, tmp_path, gpu_device):
+    """Everything at once, in bfloat16, through the entry point: prompts that share cached
+    pages, decode steps launched ahead, a pool so small that requests are preempted and
+    computed again.  Every drawn token must be a near-argmax of the plain logits."""
+    from helpers import GPU_ONLY
+    cfg, seed, page = {**TINY, **GPU_ONLY}[name]
+    d = write_random_model(tmp_path / "m", cfg, seed, torch.bfloat16,
+                           device="cpu" if name in TINY else gpu_device)
+    pcfg, w = plain.read_model_dir(d)
+    _, model = load_model(d, torch.bfloat16, gpu_device)
+    vocab = cfg["vocab_size"]
+    stem = random_prompt(2 * page + 3, vocab, 99)
+    prompts = [stem + random_prompt(n, vocab, 200 + n) for n in (1, 5, page, page + 7, 2, 9)]
+    sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+    longest = max(map(len, prompts)) + 20
+    for blocks in (64, 3 * -(-longest // page)):
+        engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page,
+                            num_kvcache_blocks=blocks, enable_prefix_caching=True,
+                            max_num_seqs=4, max_model_len=cfg["max_position_embeddings"])
+        for wave in (prompts, prompts[::-1]):
+            for prompt, completion in zip(wave, engine.generate(wave, sp, use_tqdm=False)):
+                assert len(completion) == 20
+                assert_near_greedy(pcfg, w, prompt, completion, 3e-2, 3e-2)
+        assert engine.num_steps_ahead > 0
+        assert engine.scheduler.num_prefix_hit_tokens >= 2 * page
+        if blocks != 64:
+            assert engine.scheduler.num_preemptions > 0
+        engine.runner.manager.check()
+        assert all(p.num_used == 0 for p in engine.runner.manager.pools)

@@ -57,14 +57,16 @@ def random_tensors(raw_config: dict, seed: int, dtype=torch.float32, std: float 
 
 
 def write_random_model(model_dir, raw_config: dict, seed: int, dtype=torch.float32,
-                       std: float = 0.02) -> Path:
-    """Write config.json and model.safetensors; returns the folder."""
+                       std: float = 0.02, device="cpu") -> Path:
+    """Write config.json and model.safetensors; returns the folder.  `device` is where the
+    values are drawn (a GPU draws a large model's in a second; its generator gives other
+    values than the CPU's for the same seed)."""
     model_dir = Path(model_dir)
     model_dir.mkdir(parents=True, exist_ok=True)
     cfg = dict(raw_config)
     cfg["torch_dtype"] = _DTYPE_NAMES[dtype]
-    tensors = random_tensors(cfg, seed, dtype=dtype, std=std)
+    tensors = random_tensors(cfg, seed, dtype=dtype, std=std, device=device)
     (model_dir / "config.json").write_text(json.dumps(cfg, indent=2))
-    save_file({k: v.contiguous() for k, v in tensors.items()},
+    save_file({k: v.cpu().contiguous() for k, v in tensors.items()},
               str(model_dir / "model.safetensors"))
     return model_dir
