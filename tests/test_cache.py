@@ -111,6 +111,28 @@ def test_window_release_counts_toward_what_a_step_needs():
     m.check()
 
 
+def test_shrink_undoes_an_extend():
+    from tokensprint_amd.parts.base import PagedKVNeed
+    groups, _ = group_runs([PagedKVNeed(2, 16, None), PagedKVNeed(2, 16, 8)])
+    m = CacheManager(groups, page_size=4, num_pages=12, num_slots=2)
+    rc = m.admit("a")
+    m.extend(rc, 9)
+    held = [list(t) for t in rc.tables]
+    free = [p.num_free for p in m.pools]
+    m.extend(rc, 18)                      # takes pages in both groups, the window lets one go
+    m.shrink(rc, 9)
+    assert rc.num_tokens == 9 and [len(t) for t in rc.tables] == [3, 3]
+    assert rc.tables[0] == held[0]
+    assert m.pools[0].num_free == free[0] and m.pools[1].num_free >= free[1]
+    m.check()
+    m.extend(rc, 10)                      # and goes on as if nothing had happened
+    m.check()
+    with pytest.raises(ValueError, match="cannot shrink"):
+        m.shrink(rc, 11)
+    m.free(rc)
+    assert all(p.num_used == 0 for p in m.pools)
+
+
 def test_groups_are_keyed_by_shape_and_window():
     needs = [PagedKVNeed(2, 16), PagedKVNeed(2, 16, 8), None, PagedKVNeed(2, 16),
              SlotStateNeed((4,)), PagedKVNeed(4, 16)]

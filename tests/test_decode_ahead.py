@@ -136,3 +136,42 @@ def test_a_step_ahead_is_not_launched_when_the_scheduler_has_to_decide(setup):
     while not engine.is_finished():
         engine.step()
     assert all(p.num_used == 0 for p in engine.runner.manager.pools)
+
+
+def test_a_failure_around_a_step_ahead_leaves_the_engine_usable(setup):
+    """A step launched ahead that fails (here: the runner raises) takes nothing with it:
+    the pages it took go back, nothing stays in flight, and the engine finishes the same
+    requests with the same tokens once the fault is gone."""
+    cfg, d, model, page, prompts = setup
+    L = min(cfg["max_position_embeddings"], 128)
+    sp = SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True)
+    want = engine_for(model, d, False, kvcache_block_size=page, max_model_len=L).generate(
+        prompts[:3], sp, use_tqdm=False)
+    engine = engine_for(model, d, True, kvcache_block_size=page, max_model_len=L)
+    ordinals = [engine.add_request(p, sp) for p in prompts[:3]]
+    engine.step()                       # the prompts
+    engine.step()                       # a decode step, and one launched ahead of it
+    assert engine._flight is not None and engine._flight.ahead
+    good = engine.runner.decode_and_sample
+    calls = {"n": 0}
+
+    def failing(entries, temperatures, keys, sources=None):
+        calls["n"] += 1
+        raise RuntimeError("the device refused")
+
+    engine.runner.decode_and_sample = failing
+    with pytest.raises(RuntimeError, match="refused"):
+        engine.step()                   # finishes the step in flight, fails launching ahead
+    assert calls["n"] == 1 and engine._flight is None
+    engine.runner.manager.check()
+    for req in engine.scheduler.running:            # each holds its tokens' pages, no more
+        assert len(req.cache.tables[0]) == -(-req.cache.num_tokens // page)
+    engine.runner.decode_and_sample = good
+    # the step that was in flight when the launch failed is lost with its tokens (its
+    # requests are one token short and compute it again): same tokens in the end
+    outputs = {}
+    while not engine.is_finished():
+        for ordinal, tokens in engine.step()[0]:
+            outputs[ordinal] = tokens
+    assert [outputs[o] for o in ordinals] == want
+    assert all(p.num_used == 0 for p in engine.runner.manager.pools)

@@ -53,7 +53,7 @@ def test_prefill_then_decode(setup):
 
 def test_mixed_with_page_reuse(setup):
     model, requests, ref, (rtol, atol) = setup
-    # pages for 128 of the 145 tokens: the short requests' pages serve the long one's end
-    runner = ModelRunner(model, page_size=PAGE, num_pages=128 // PAGE, num_slots=4)
+    # ten pages where the three requests need 1 + 3 + 7: the shortest one's page is used again
+    runner = ModelRunner(model, page_size=PAGE, num_pages=10, num_slots=4)
     drives.compare(drives.drive_mixed(runner, requests), ref, rtol, atol)
     assert all(pool.num_used == 0 for pool in runner.manager.pools)

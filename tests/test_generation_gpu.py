@@ -282,7 +282,7 @@ def test_bfloat16_with_prefix_cache_steps_ahead_and_preemption(name, tmp_path, g
     prompts = [stem + random_prompt(n, vocab, 200 + n) for n in (1, 5, page, page + 7, 2, 9)]
     sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
     longest = max(map(len, prompts)) + 20
-    for blocks in (64, 3 * -(-longest // page)):
+    for blocks in (64, 2 * -(-longest // page)):
         engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page,
                             num_kvcache_blocks=blocks, enable_prefix_caching=True,
                             max_num_seqs=4, max_model_len=cfg["max_position_embeddings"])

@@ -643,6 +643,55 @@ def test_decode_kernel_merges_its_key_splits_as_the_merge_kernel_does(ops, gpu_d
         assert torch.equal(out, apart)
 
 
+def test_decode_kernel_merge_over_hundreds_of_launches(ops, gpu_device, monkeypatch):
+    """The in-kernel merge rests on an order of memory operations (partial results by
+    device-scope stores that each wave waits for, then the count; the last workgroup reads
+    them back by device-scope loads).  Hundreds of launches back to back over many items
+    (24 entries x 8 heads, two to five splits each, contexts that change from launch to
+    launch), with other kernels' traffic between them, each compared bit for bit with the
+    merge kernel's result; stops at the first launch that differs."""
+    dtype, page, nq, nkv, hd = torch.bfloat16, 16, 16, 8, 128
+    g = torch.Generator().manual_seed(5)
+    cases = []
+    for n in (3, 24, 9):
+        spans = [(int(torch.randint(130, 3000, (1,), generator=g)), 1) for _ in range(n)]
+        batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd,
+                                                page_size=page, spans=spans, seed=90 + n)
+        assert ops._decode_splits(n * nkv, batch.max_ctx_len) > 1
+        qkv = rand((batch.num_tokens, (nq + 2 * nkv) * hd), dtype, gpu_device, 91 + n)
+        cases.append((batch, cache, table, qkv))
+    wq = 1 + 0.1 * rand((hd,), torch.float32, gpu_device, 73)
+    angles = torch.outer(torch.arange(3100, dtype=torch.float32),
+                         1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    cos_sin = (angles.cos().to(gpu_device), angles.sin().to(gpu_device))
+    kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, q_weight=wq, k_weight=wq, eps=1e-6,
+              cos_sin=cos_sin, scale=hd ** -0.5, window=None, kv_in_row=nkv)
+    monkeypatch.setattr(ops, "fold_merge", False)
+    apart = [ops.attend(qkv, batch, table, cache, True, **kw).clone()
+             for batch, cache, table, qkv in cases]
+    monkeypatch.setattr(ops, "fold_merge", True)
+    filler = rand((4096, 4096), torch.float32, gpu_device, 7)
+    outs = []
+    for launch in range(240):
+        batch, cache, table, qkv = cases[launch % 3]
+        outs.append(ops.attend(qkv, batch, table, cache, True, **kw))
+        if launch % 4 == 0:
+            filler.mul_(1.0)                   # other traffic through the caches
+        if launch % 40 == 39:                  # compared in groups: the launches stay back to back
+            for k, out in enumerate(outs):
+                assert torch.equal(out, apart[(launch - 39 + k) % 3]), \
+                    f"launch {launch - 39 + k} differs from the merge kernel's result"
+            outs.clear()
+    assert int(ops._arrivals.abs().sum()) == 0
+    # counts left behind by a launch that did not finish would make later merges wrong:
+    # `reset_scratch` (after every failed call, before warm-up and capture) clears them
+    ops._arrivals[:5] = 3
+    ops.reset_scratch()
+    assert int(ops._arrivals.abs().sum()) == 0
+    batch, cache, table, qkv = cases[1]
+    assert torch.equal(ops.attend(qkv, batch, table, cache, True, **kw), apart[1])
+
+
 @pytest.mark.parametrize("window", [None, 1000])
 @pytest.mark.parametrize("fused", [True, False])
 def test_attend_decode_long_contexts_split_and_merge(ops, gpu_device, window, fused):

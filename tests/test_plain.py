@@ -82,6 +82,30 @@ def test_rope_scores_depend_on_distance_only_and_sign_is_right():
     torch.testing.assert_close(y[0, 0, 8], torch.tensor(math.sin(1.0)))
 
 
+def test_rope_is_a_complex_multiplication():
+    # The rotate-half form of engine/kernels/triton/rope.py:53-65 and engine/nn/rope.py:
+    # element i and element i + hd/2 are the real and imaginary part of one complex
+    # number, multiplied by exp(i * pos * inv_freq[i]).  Written with the library's complex
+    # arithmetic, which knows nothing of halves, signs or tables; the interleaved pairing
+    # (2i, 2i+1) and the conjugate rotation both fail it.
+    hd, theta = 32, 1e4
+    x = rnd(7, 3, hd, seed=5)
+    pos = torch.tensor([0, 1, 2, 17, 100, 211, 300])     # (float32 angles: pos * 6e-8 of error)
+    cos, sin = plain.rope_cos_sin(pos, hd, theta)
+    got = plain.apply_rope(x, cos, sin)
+    z = torch.complex(x[..., :hd // 2].double(), x[..., hd // 2:].double())
+    freq = theta ** (-torch.arange(0, hd, 2, dtype=torch.float64) / hd)
+    turn = torch.polar(torch.ones(7, hd // 2, dtype=torch.float64), pos[:, None].double() * freq)
+    want = z * turn[:, None, :]
+    torch.testing.assert_close(got[..., :hd // 2].double(), want.real, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(got[..., hd // 2:].double(), want.imag, rtol=1e-4, atol=1e-4)
+    other = z * turn.conj()[:, None, :]
+    assert (got[..., hd // 2:].double() - other.imag).abs().max() > 0.1
+    zi = torch.view_as_complex(x.double().reshape(7, 3, hd // 2, 2).contiguous()) * turn[:, None, :]
+    interleaved = torch.view_as_real(zi).reshape(7, 3, hd)
+    assert (got.double() - interleaved).abs().max() > 0.1
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("nq,nkv", [(4, 4), (8, 2), (6, 3), (1, 1)])
 def test_attention_is_the_library_routine(nq, nkv):

@@ -335,6 +335,22 @@ class CacheManager:
                 table.append(self.pools[g].take())
         rc.num_tokens = new_len
 
+    def shrink(self, rc: RequestCache, new_len: int) -> None:
+        """Undo an `extend` whose tokens will not be computed after all: the request holds
+        `new_len` tokens again and the pages beyond them go back.  (Pages a window let go
+        on the way stay gone: no query from `new_len` on could see them.)"""
+        if new_len > rc.num_tokens:
+            raise ValueError(f"cannot shrink a request from {rc.num_tokens} to {new_len}")
+        if new_len < len(rc.hashes) * self.page_size:
+            raise ValueError("cannot shrink a request into its registered pages")
+        total = -(-new_len // self.page_size)
+        for g, table in enumerate(rc.tables):
+            while len(table) > max(total, rc.released[g]):
+                page = table.pop()
+                if page >= 0:
+                    self.pools[g].give_back(page)
+        rc.num_tokens = new_len
+
     def release_passed(self, rc: RequestCache) -> None:
         """Give back the pages no query at position >= rc.num_tokens can see."""
         for g, table in enumerate(rc.tables):

@@ -49,6 +49,8 @@ class Config:
     enable_prefix_caching: bool = False   # share cached full pages between equal prefixes
     warmup: bool = True                   # largest dummy step and graph capture at construction
     decode_ahead: bool = True             # launch a decode step before the last one's tokens are read
+    fold_merge: bool = True               # a decode step's attention merges its key splits itself
+                                          # (False: a merge kernel of its own after it)
 
     def __post_init__(self) -> None:
         if not os.path.isdir(self.model):

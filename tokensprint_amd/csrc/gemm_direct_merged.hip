@@ -22,11 +22,14 @@ int gemm_direct_merged(const DirectArgs& a, hipStream_t stream) {
 }
 
 // Whether ts_gemm_tail_merged_bf16 takes this product: what the tail form takes, one
-// tile of rows, whole 8-element pieces inside a head, rows that fit LDS.
+// tile of rows, whole 8-element pieces inside a head, and the merged rows of A (as
+// launch_merged lays them out, padded to the rows a load is packed for) within the 160 KiB
+// of LDS a workgroup can have.
 extern "C" int ts_gemm_tail_merged_fits(int M, int N, int heads, int hd) {
   const int64_t K = (int64_t)heads * hd;
-  return M >= 1 && M <= 16 && heads >= 1 && hd >= 8 && hd % 8 == 0 && K <= 8192 &&
-         gemm_direct_tail_fits(M, N, (int)K);
+  if (!(M >= 1 && M <= 16 && heads >= 1 && hd >= 8 && hd % 8 == 0 && K <= 8192)) return 0;
+  const int64_t lds = (int64_t)gemm_direct_packed_rows(M) * (K / 8 + 1) * 16;
+  return lds <= 160 * 1024 && gemm_direct_tail_fits(M, N, (int)K);
 }
 
 // Rows up to which it pays.  Every workgroup merges all rows, and what it reads for that

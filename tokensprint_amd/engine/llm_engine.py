@@ -47,6 +47,8 @@ class LLMEngine:
         page = config.kvcache_block_size
         on_gpu = model.ctx.device.type == "cuda"
         graph_len = None if config.enforce_eager or not on_gpu else config.max_model_len
+        if hasattr(model.ctx.ops, "fold_merge"):
+            model.ctx.ops.fold_merge = bool(config.fold_merge)
         # the shapes that the warm-up meets (the largest step, the captured decode steps)
         # are the ones the run is made of: their library plans are worth timing
         timed_plans = getattr(model.ctx.ops, "timed_plans", lambda on: False)
@@ -190,8 +192,29 @@ class LLMEngine:
         flight = self._flight or self._launch(self.scheduler.schedule())
         self._flight = None
         if flight.event is not None and self.config.decode_ahead:
-            self._flight = self._launch_ahead(flight)
-        return self._finish(flight)
+            try:
+                self._flight = self._launch_ahead(flight)
+            except BaseException:
+                self._give_back_pages_taken_ahead(flight)
+                raise
+        try:
+            return self._finish(flight)
+        except BaseException:
+            # the step that was launched ahead dies with the one it follows: nobody will
+            # read its tokens, and the pages it took go back
+            if self._flight is not None:
+                self._give_back_pages_taken_ahead(flight)
+                self._flight = None
+            raise
+
+    def _give_back_pages_taken_ahead(self, prev: _Flight) -> None:
+        """After a failure around a step launched ahead of `prev`: every request of `prev`
+        that still runs holds exactly the pages of the tokens it has and the one `prev`
+        computes, as if nothing had been launched ahead."""
+        manager = self.runner.manager
+        for req, pos in zip(prev.reqs, prev.positions or []):
+            if req.status is RequestStatus.RUNNING and req.cache is not None:
+                manager.shrink(req.cache, pos + 1)
 
     def _land(self, drawn: torch.Tensor):
         """Enqueue the copy of a captured step's tokens to the host."""

@@ -133,10 +133,18 @@ class ModelRunner:
         """Capture every decode bucket now, the largest first so that the smaller ones fit
         into the memory it took (engine/generation/model_runner.py:334,373-379 captures in
         that order for that reason).  Without this a bucket is captured at its first use."""
+        self._reset_provider()
         self._choose_large_weight_rows()
         for bucket in reversed(self.buckets):
             if bucket not in self.graphs:
                 self._capture(bucket)
+
+    def _reset_provider(self) -> None:
+        """What the kernel provider keeps between calls, back to its start (a provider
+        without such state has no `reset_scratch`)."""
+        reset = getattr(self.model.ctx.ops, "reset_scratch", None)
+        if reset is not None:
+            reset()
 
     def _choose_large_weight_rows(self) -> None:
         """Where the kernel provider has a choice to offer for the products of few rows
@@ -196,6 +204,7 @@ class ModelRunner:
             manager.extend(rc, per)
             entries.append(StepEntry(rc, [0] * per, 0, [per - 1]))
         try:
+            self._reset_provider()
             self.run(self.build(entries))
             if self.device.type == "cuda":
                 torch.cuda.synchronize(self.device)

@@ -117,7 +117,10 @@ class HipOps:
         self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
         # Above those rows the decode kernel merges its key splits itself: the workgroups of
         # an item count themselves in here and the last one merges.  The kernel leaves every
-        # count at zero, so one zeroed array serves every launch (of one stream).
+        # count at zero, so one zeroed array serves every launch (of one stream); a launch
+        # that did not run to its end may leave counts behind, so the array is zeroed again
+        # after every failed call and before warm-up and capture (`reset_scratch`).
+        # `fold_merge = False` gives the merge a kernel of its own again.
         self.fold_merge = True
         self._arrivals = torch.zeros(4096, dtype=torch.int32, device=self.device)
 
@@ -128,7 +131,17 @@ class HipOps:
 
     def _call(self, fn, *args):
         if fn(*args) != 0:
-            raise KernelError(self.lib.ts_last_error().decode())
+            message = self.lib.ts_last_error().decode()
+            self.reset_scratch()
+            raise KernelError(message)
+
+    def reset_scratch(self) -> None:
+        """Put what this provider keeps between calls back to its start: the arrival counts
+        of the decode kernel's own merge at zero, no deferred merge pending.  Called after a
+        failed call, and by the engine before its warm-up step and before graphs are
+        captured."""
+        self._unmerged = None
+        self._arrivals.zero_()
 
     def _check(self, name, t, dtype=None, shape=None, ndim=None):
         # (written for the case that all is well, which is every call of a working engine:
@@ -428,18 +441,20 @@ class HipOps:
                 or self.lib.ts_gemm_tail_merged_fits(M, N, a.nq, a.hd) != 1 \
                 or self.lib.ts_gemm_scaled_fits(M, next_n, N, int(hint.silu_mul), parts) != 1:
             return None
-        self._unmerged = None
         self._check("weight", weight, torch.bfloat16, ndim=2)
         self._check("resid", resid, torch.float32, shape=(M, N))
         self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
         rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
         sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
+        # (the merge stays pending until the kernel that does it has been launched: a refusal
+        # raises, and a failed call clears it with the rest of the scratch state)
         self._call(self.lib.ts_gemm_tail_merged_bf16, _ptr(unmerged.partial_o),
                    _ptr(unmerged.partial_ml), _ptr(unmerged.positions),
                    unmerged.args.num_splits, a.nq, a.nkv, a.hd,
                    0 if unmerged.window is None else int(unmerged.window), _ptr(weight),
                    _ptr(resid), _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N,
                    self._stream())
+        self._unmerged = None
         return PreparedRows(rows, sumsq, hint)
 
     def _prepared_linear(self, resid, prepared, norm_weight, eps, weight, out_dtype, silu_mul):
@@ -807,6 +822,14 @@ class HipOps:
         `longest_first`: sorted by the number of keys a run's last token sees, most first
         (the kernels for long portions pair runs from both ends of that order)."""
         key = ("attn_tiles", tokens, longest_first)
+        if key not in batch.plans and batch.max_q_len == 1:
+            # a step of single tokens: tile i is entry i.  No order: the host's `starts` of a
+            # captured decode batch are placeholders, and the order is a hint for the
+            # kernel's balance only, never for what it computes (it reads positions and
+            # lengths on the device).
+            tiles = [(entry, entry, 1) for entry in range(batch.num_entries)]
+            host = torch.tensor(tiles, dtype=torch.int32)
+            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
         if key not in batch.plans:
             tiles, keys = [], []
             first = 0
