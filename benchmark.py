@@ -46,6 +46,8 @@ def parse_args(argv=None):
     ap.add_argument("--use-tqdm", type=_bool, default=True)
     ap.add_argument("--max-prompt-token-id", type=int, default=10000)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--cast-weights", type=_bool, default=False,
+                    help="with --model-dir, bfloat16: round 32-bit matrices to bfloat16")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=-1)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers (random weights only)")
@@ -77,7 +79,7 @@ def main(args) -> None:
     seed(0)
     prompts, output_lens = make_workload(args)
     if args.model_dir is not None:
-        _, model = load_model(args.model_dir, args.dtype, "cuda:0")
+        _, model = load_model(args.model_dir, args.dtype, "cuda:0", cast_32bit=args.cast_weights)
         model_dir = str(args.model_dir)
     else:
         raw = json.loads(args.config_json.read_text()) if args.config_json is not None \

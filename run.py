@@ -48,6 +48,9 @@ def parse_args(argv=None):
                     help="with --random-weights: this config.json instead of --model-name's")
     ap.add_argument("--prompt-ids", default=None,
                     help="comma-separated token ids instead of --prompt (no tokenizer needed)")
+    ap.add_argument("--cast-weights", type=_bool, default=False,
+                    help="bfloat16 run: round matrices the checkpoint stores in 32-bit to "
+                         "bfloat16 (default: they stay 32-bit, on the float32 kernels)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=-1)
     ap.add_argument("--max-num-batched-tokens", type=int, default=16384)
@@ -83,7 +86,7 @@ def main(args) -> None:
         raise ValueError("--config-json describes random weights: give --random-weights SEED")
     elif model_dir is None:
         model_dir = args.cache_dir / get_model_repo_id(args.model_name).split("/")[-1]
-    _, model = load_model(model_dir, dtype, "cuda:0")
+    _, model = load_model(model_dir, dtype, "cuda:0", cast_32bit=args.cast_weights)
     spec = model.spec           # sizes and the end-of-sequence token come from the model as
                                 # built, whatever architecture config.json named
 

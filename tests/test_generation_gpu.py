@@ -224,7 +224,8 @@ def test_warm_up_chooses_who_multiplies_large_weights(setup, gpu_device, tmp_pat
     pcfg, w = plain.read_model_dir(d)
     _, model = load_model(d, torch.bfloat16, gpu_device)
     ops = model.ctx.ops
-    monkeypatch.setattr(ops, "LARGE_WEIGHT", 1 << 8)
+    import dataclasses
+    monkeypatch.setattr(ops, "dispatch", dataclasses.replace(ops.dispatch, large_weight=1 << 8))
     monkeypatch.setattr(ops, "_large_rows", {})
     monkeypatch.setattr(ops, "_large_undecided", set())
     L = cfg["max_position_embeddings"]

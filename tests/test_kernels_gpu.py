@@ -114,10 +114,10 @@ def test_linear(ops, gpu_device, x_dtype, w_dtype, out_dtype, M, N, K):
     w = rand((N, K), w_dtype, gpu_device, 8, scale=0.1)
     out = ops.linear(x, w, out_dtype)
     ref = x.double() @ w.double().T
-    # the vendor library's result is bfloat16 also when float32 is asked for
-    widened = x_dtype == w_dtype == torch.bfloat16 and from_library(M, N, K)
-    t = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 and not widened \
-        else dict(rtol=1e-2, atol=1e-2)
+    # every kernel sums in float32, the vendor library's too, and a float32 result leaves
+    # unrounded: held to float32 rounding whatever the operands' types; a bfloat16 result
+    # to bfloat16's
+    t = dict(rtol=1e-5, atol=1e-5) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(out.double(), ref, **t)
 
 
@@ -241,7 +241,7 @@ def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
         first = out if first is None else first
         assert torch.equal(out, first), f"tile {tile} differs"
     # the engine's entry takes this kernel from 65 rows on at weights of this size
-    if 2 * I * K <= ops.TILED_PAIR_WEIGHT:
+    if 2 * I * K <= ops.dispatch.tiled_pair_weight:
         assert torch.equal(ops.linear_silu_mul(x, w, torch.bfloat16), first)
 
 
@@ -647,13 +647,13 @@ def test_decode_kernel_merge_over_hundreds_of_launches(ops, gpu_device, monkeypa
     """The in-kernel merge rests on an order of memory operations (partial results by
     device-scope stores that each wave waits for, then the count; the last workgroup reads
     them back by device-scope loads).  Hundreds of launches back to back over many items
-    (24 entries x 8 heads, two to five splits each, contexts that change from launch to
+    (up to 16 entries x 8 heads, two to ten splits each, contexts that change from launch to
     launch), with other kernels' traffic between them, each compared bit for bit with the
     merge kernel's result; stops at the first launch that differs."""
     dtype, page, nq, nkv, hd = torch.bfloat16, 16, 16, 8, 128
     g = torch.Generator().manual_seed(5)
     cases = []
-    for n in (3, 24, 9):
+    for n in (3, 16, 9):
         spans = [(int(torch.randint(130, 3000, (1,), generator=g)), 1) for _ in range(n)]
         batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd,
                                                 page_size=page, spans=spans, seed=90 + n)
@@ -743,7 +743,7 @@ def test_output_projection_merges_the_key_splits_itself(ops, gpu_device, monkeyp
     Stream, prepared rows and sums of squares must be, bit for bit, what the merge kernel
     followed by the tail form leaves; and a deferred merge that another call meets (a
     plain product here) is run before that call."""
-    from tokensprint_amd.kernels.stream import NormHint
+    from tokensprint_amd.kernels.stream import NormHint, UnmergedRows
     dtype, page = torch.bfloat16, 16
     batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
                                             spans=spans, seed=81)
@@ -770,10 +770,11 @@ def test_output_projection_merges_the_key_splits_itself(ops, gpu_device, monkeyp
         mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
                            cache.k_pages.clone(), cache.v_pages.clone())
         o = ops.attend(qkv, batch, table, mine, True, defer_merge=defer, **kw).view(T, nq * hd)
-        assert (ops._unmerged is not None) == defer
+        assert isinstance(o, UnmergedRows) == defer and tuple(o.shape) == (T, nq * hd)
         resid = resid0.clone()
         prepared = ops.linear_into_stream(o, w_o, resid, hint)
-        assert ops._unmerged is None
+        if defer:
+            assert not o.is_merged          # the product's kernel merged the rows itself
         return o, resid, prepared
 
     o_ref, resid_ref, prep_ref = run(False)
@@ -787,9 +788,16 @@ def test_output_projection_merges_the_key_splits_itself(ops, gpu_device, monkeyp
                        cache.k_pages.clone(), cache.v_pages.clone())
     o = ops.attend(qkv, batch, table, mine, True, defer_merge=True, **kw).view(T, nq * hd)
     y = ops.linear(o, w_o, dtype)
-    assert ops._unmerged is None
-    assert torch.equal(o, o_ref)
+    assert o.is_merged
+    assert torch.equal(o.merged(), o_ref)
     assert torch.equal(y, ops.linear(o_ref, w_o, dtype))
+    # the handle is no tensor: code that is not this provider's cannot read unmerged rows
+    o = ops.attend(qkv, batch, table, mine, True, defer_merge=True, **kw)
+    with pytest.raises(TypeError):
+        torch.matmul(o, w_o.T)
+    with pytest.raises(TypeError, match="unmerged"):
+        ops.silu_mul(o.view(T, nq * hd))
+    assert torch.equal(o.view(T, nq * hd).merged(), o_ref)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -13,9 +13,10 @@ from tokensprint_amd.engine import ModelRunner, StepEntry
 from tokensprint_amd.engine.assemble import random_model
 from tokensprint_amd.engine.batch import BatchBuilder
 from tokensprint_amd.models.spec import LayerSpec, ModelSpec, PartSpec, Run
-from tokensprint_amd.parts import (FEED_FORWARDS, MIXERS, POSITIONS, BuildContext, FeedForward,
-                                   Mixer, PositionEncoding, SlotStateNeed, TensorDecl,
-                                   build_part, register, NORMS, BLOCKS)
+from tokensprint_amd.parts import (EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, POSITIONS, Block,
+                                   BuildContext, Embedding, FeedForward, Head, Mixer,
+                                   PositionEncoding, SlotStateNeed, TensorDecl, build_part,
+                                   register, NORMS, BLOCKS)
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
@@ -111,7 +112,8 @@ def test_attention_and_swiglu_and_block_parts(gpu_device, dtype, window):
     ref_ffn = plain.swiglu(h.float(), w, "f.")
     torch.testing.assert_close(ffn.forward(h.to(gpu_device), batch).float().cpu(), ref_ffn, **tol(dtype))
     # the block: x + attn(norm(x)), then + ffn(norm(.))
-    block = BLOCKS["pre_norm"](mixer, ffn, n1, n2, ctx)
+    block = BLOCKS["pre_norm"]({"mixer": mixer, "feed_forward": ffn, "mixer_norm": n1,
+                                "ffn_norm": n2}, ctx)
     x = rnd((T, width), 6)
     resid, delta = block.forward(x.to(gpu_device), None, batch, storage.views[0], True)
     x1 = x + plain.attention_mixer(plain.rms_norm(x, w["n1"], 1e-6).to(dtype).float(), pw, "a.",
@@ -217,6 +219,34 @@ class ToyOffsetEncoding(PositionEncoding):
             k.copy_((k.float() + shift).to(k.dtype))
 
 
+class ToyScaledEmbedding(Embedding):
+    """Rows of the table times a constant (as architectures that scale their embeddings by
+    the root of the width do)."""
+
+    def forward(self, token_ids):
+        return super().forward(token_ids) * self.params["scale"]
+
+
+class ToyCappedHead(Head):
+    """Logits squashed into (-cap, cap): cap * tanh(logits / cap)."""
+
+    def forward_from_stream(self, resid, delta, norm):
+        cap = self.params["cap"]
+        return cap * torch.tanh(super().forward_from_stream(resid, delta, norm) / cap)
+
+
+class ToySandwichBlock(Block):
+    """A layer without a feed-forward whose mixer sits between two norms:
+    x = x + post_norm(mixer(mixer_norm(x)))."""
+
+    ROLES = {"mixer_norm": (NORMS, True), "mixer": (MIXERS, True), "post_norm": (NORMS, True)}
+
+    def forward(self, resid, delta, batch, cache, write_cache, next_hint=None):
+        h = self.mixer_norm.forward(resid) if delta is None \
+            else self.mixer_norm.add_forward(resid, delta)
+        return resid, self.post_norm.forward(self.mixer.forward(h, batch, cache, write_cache))
+
+
 def toy_spec(raw):
     W, V = raw["width"], raw["vocab"]
     norm = lambda name: PartSpec("rmsnorm", {"dim": W, "eps": 1e-5, "weight": name})
@@ -231,16 +261,23 @@ def toy_spec(raw):
                   PartSpec("toy_top1", {"prefix": "l1.ffn."}), norm("l1.n1"), norm("l1.n2")),
         LayerSpec("pre_norm", attn("l2.attn.", "rope", own=False), PartSpec("swiglu", {"prefix": "l2.ffn.", "inner_dim": 24}),
                   norm("l2.n1"), norm("l2.n2")),
+        # a block kind of the test's own: no feed-forward, a norm behind the mixer
+        LayerSpec("toy_sandwich", mixer=attn("l3.attn.", "rope"), mixer_norm=norm("l3.n1"),
+                  post_norm=norm("l3.post")),
+        # and a pre-norm layer that is a feed-forward only: its run owns no cache
+        LayerSpec("pre_norm", feed_forward=PartSpec("swiglu", {"prefix": "l4.ffn.", "inner_dim": 56}),
+                  ffn_norm=norm("l4.n2")),
     )
     return ModelSpec(
         architecture="ToyForTests", width=W, vocab_size=V,
-        embedding=PartSpec("embedding", {"weight": "embed", "vocab_size": V}),
+        embedding=PartSpec("toy_scaled_embedding", {"weight": "embed", "vocab_size": V, "scale": 3.0}),
         positions={"offset": PartSpec("toy_offset", {"step": 0.01}),
                    "rope": PartSpec("rope", {"dim": 16, "theta": 100.0, "max_position": 128})},
         layers=layers,
         # layer 0 runs twice (two caches of its own); layer 2 reads the cache of run 0
-        order=(Run(0), Run(1), Run(0), Run(2, cache_of=0)),
-        final_norm=norm("final"), head=PartSpec("head", {"weight": "embed", "vocab_size": V, "tied": True}),
+        order=(Run(0), Run(1), Run(0), Run(2, cache_of=0), Run(3), Run(4)),
+        final_norm=norm("final"),
+        head=PartSpec("toy_capped_head", {"weight": "embed", "vocab_size": V, "tied": True, "cap": 2.0}),
         max_position=128)
 
 
@@ -249,7 +286,10 @@ def toy_registered():
     for reg, kind, cls in ((MIXERS, "toy_decay", ToyDecayMixer),
                            (MIXERS, "toy_decay_on_device", ToyDecayMixerOnDevice),
                            (FEED_FORWARDS, "toy_top1", ToyTop1FeedForward),
-                           (POSITIONS, "toy_offset", ToyOffsetEncoding)):
+                           (POSITIONS, "toy_offset", ToyOffsetEncoding),
+                           (EMBEDDINGS, "toy_scaled_embedding", ToyScaledEmbedding),
+                           (HEADS, "toy_capped_head", ToyCappedHead),
+                           (BLOCKS, "toy_sandwich", ToySandwichBlock)):
         register(reg, kind, replace=True)(cls)
     if "ToyForTests" not in _ARCHITECTURES:
         register_architecture("ToyForTests", parse_config=lambda raw: raw, build_spec=toy_spec)
@@ -262,7 +302,7 @@ def toy_plain(model, tokens):
     b = model.blocks
     T = len(tokens)
     pos = torch.arange(T)
-    x = g(model.embedding.table)[tokens]
+    x = 3.0 * g(model.embedding.table)[tokens]
 
     def attention(blk, h, k_src, mode):
         m = blk.mixer
@@ -277,7 +317,12 @@ def toy_plain(model, tokens):
         else:
             cos, sin = plain.rope_cos_sin(pos, 16, 100.0)
             q = plain.apply_rope(q, cos, sin)
-            k, v = k_src
+            if k_src is None:          # a layer with keys of its own behind the rotation
+                k = plain.apply_rope(plain.rms_norm(qkv[:, 64:96].view(T, 2, 16), g(m.w_knorm), 1e-5),
+                                     cos, sin)
+                v = qkv[:, 96:].view(T, 2, 16)
+            else:
+                k, v = k_src
         o = plain.causal_attention(q, k, v)
         return o.reshape(T, 64) @ g(m.w_o).T, (k, v)
 
@@ -307,15 +352,20 @@ def toy_plain(model, tokens):
     a, _ = attention(b[2], norm(b[2].mixer_norm, x), kv0, "rope")                # run 3 reads run 0's cache
     x = x + a
     x = x + swiglu(b[2], norm(b[2].ffn_norm, x))
-    return norm(model.final_norm, x) @ g(model.embedding.table).T
+    a, _ = attention(b[3], norm(b[3].mixer_norm, x), None, "rope")               # run 4: the sandwich
+    x = x + norm(b[3].post_norm, a)
+    assert b[3].parts() == [b[3].mixer_norm, b[3].mixer, b[3].post_norm] and b[4].mixer is None
+    x = x + swiglu(b[4], norm(b[4].ffn_norm, x))                                 # run 5: feed-forward only
+    return 2.0 * torch.tanh(norm(model.final_norm, x) @ g(model.embedding.table).T / 2.0)
 
 
 def test_toy_parts_build_and_step(toy_registered, gpu_device):
     _, model = random_model(toy_registered, seed=5, dtype=torch.float32, device=gpu_device, std=0.2)
     needs = model.cache_needs()
-    assert [type(n).__name__ for n in needs] == ["PagedKVNeed", "SlotStateNeed", "PagedKVNeed", "NoneType"]
+    assert [type(n).__name__ for n in needs] == ["PagedKVNeed", "SlotStateNeed", "PagedKVNeed", "NoneType",
+                                                 "PagedKVNeed", "NoneType"]
     runner = ModelRunner(model, page_size=4, num_pages=40, num_slots=3)
-    assert len(runner.storage.groups) == 1 and runner.storage.groups[0].runs == (0, 2)
+    assert len(runner.storage.groups) == 1 and runner.storage.groups[0].runs == (0, 2, 4)
     assert runner.storage.views[1].state.shape == (3 + 1, 64)     # one row for idle lanes
     g = torch.Generator().manual_seed(0)
     reqs = {rid: torch.randint(0, 97, (n,), generator=g).tolist() for rid, n in (("a", 30), ("b", 19), ("c", 44))}

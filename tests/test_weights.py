@@ -87,6 +87,26 @@ def test_bf16_run_keeps_32bit_tensors(tmp_path):
     assert model.blocks[0].mixer_norm.weight.dtype == torch.float32
 
 
+def test_bf16_run_warns_about_32bit_matrices_and_can_round_them(tmp_path, caplog):
+    d = write_random_model(tmp_path / "m", TINY_B, 1, torch.float32)
+    with caplog.at_level("WARNING"):
+        _, model = load_model(d, "bfloat16", "cpu", ops=TorchOps())
+    assert model.blocks[0].feed_forward.w_down.dtype == torch.float32
+    assert "stay so in this bfloat16 run" in caplog.text and "cast_32bit=True" in caplog.text
+    caplog.clear()
+    with caplog.at_level("WARNING"):
+        _, model = load_model(d, "bfloat16", "cpu", ops=TorchOps(), cast_32bit=True)
+    assert not caplog.text
+    assert model.blocks[0].feed_forward.w_down.dtype == torch.bfloat16
+    assert model.embedding.table.dtype == torch.bfloat16
+    assert model.blocks[0].mixer_norm.weight.dtype == torch.float32       # vectors stay float32
+    ref = load_file(str(d / "model.safetensors"))["model.layers.0.mlp.down_proj.weight"]
+    assert torch.equal(model.blocks[0].feed_forward.w_down, ref.to(torch.bfloat16))
+    # a float32 run holds everything in float32 whatever is asked
+    _, model = load_model(d, "float32", "cpu", ops=TorchOps(), cast_32bit=True)
+    assert model.blocks[0].feed_forward.w_down.dtype == torch.float32
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     d = write_random_model(tmp_path / "m", TINY_B, 1, torch.float32)
     t = load_file(str(d / "model.safetensors"))

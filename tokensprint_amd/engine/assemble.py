@@ -45,10 +45,12 @@ def build_model(raw_config: dict, dtype, device, ops=None):
     return config, Model(spec, ctx)
 
 
-def load_model(model_dir, dtype="bfloat16", device="cuda:0", ops=None):
-    """(typed config, Model with weights) from a folder with config.json and safetensors."""
+def load_model(model_dir, dtype="bfloat16", device="cuda:0", ops=None, cast_32bit=False):
+    """(typed config, Model with weights) from a folder with config.json and safetensors.
+    `cast_32bit`: in a bfloat16 run, round matrices the files store in 32-bit to bfloat16
+    (by default they stay 32-bit and are served by the float32 kernels)."""
     config, model = build_model(read_config_json(model_dir), dtype, device, ops)
-    load_weights(model, model_dir, model.ctx.dtype, model.ctx.device)
+    load_weights(model, model_dir, model.ctx.dtype, model.ctx.device, cast_32bit=cast_32bit)
     return config, model
 
 

@@ -164,7 +164,8 @@ class LLMEngine:
             raise ValueError("a text prompt needs a tokenizer; pass token ids instead")
         token_ids = self.tokenizer.encode(prompt, add_special_tokens=True)
         if not isinstance(token_ids, list):
-            raise TypeError("Expected tokenizer.encode(...) to return list[int].")
+            raise TypeError(f"the tokenizer's encode gave {type(token_ids).__name__}, "
+                            "a list of token ids is needed")
         return token_ids
 
     def is_finished(self) -> bool:
@@ -312,8 +313,8 @@ class LLMEngine:
         if not isinstance(sampling_params, list):
             sampling_params = [sampling_params] * len(prompts)
         if len(sampling_params) != len(prompts):
-            raise ValueError("sampling_params length must match prompts length, "
-                             f"got {len(sampling_params)} and {len(prompts)}.")
+            raise ValueError(f"{len(prompts)} prompts but {len(sampling_params)} sampling "
+                             "parameters: give one for all, or a list of equal length")
         pbar = None
         if use_tqdm:
             from tqdm.auto import tqdm

@@ -51,8 +51,9 @@ class Scheduler:
     def add_request(self, req: Request) -> None:
         if len(req) > self.max_model_len - 1:
             raise ValueError(
-                "Sequence length exceeds max_model_len: "
-                f"got {len(req)}, max allowed is {self.max_model_len - 1}.")
+                f"a request of {len(req)} tokens is too long: with max_model_len="
+                f"{self.max_model_len} at most {self.max_model_len - 1} fit before the first "
+                "generated token")
         need = -(-(len(req) + 1) // self.manager.page_size)
         full = [pool.num_pages for g, pool in zip(self.manager.groups, self.manager.pools)
                 if g.window is None]
@@ -162,8 +163,8 @@ class Scheduler:
                     sampled_index: list[int]) -> None:
         """`token_ids[i]` was drawn for `reqs[sampled_index[i]]`."""
         if len(token_ids) != len(sampled_index):
-            raise ValueError("token_ids and sampled_index must have equal length, "
-                             f"got {len(token_ids)} and {len(sampled_index)}.")
+            raise ValueError(f"{len(token_ids)} drawn tokens for {len(sampled_index)} "
+                             "requests that were to draw one")
         for req in reqs:
             req.num_cached_tokens += req.num_new_tokens
             req.num_new_tokens = 0

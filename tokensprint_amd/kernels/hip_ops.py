@@ -14,7 +14,8 @@ from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
 import torch
 
 from tokensprint_amd.kernels.build import build, find_library
-from tokensprint_amd.kernels.stream import NormHint, PreparedRows
+from tokensprint_amd.kernels.dispatch import default_dispatch
+from tokensprint_amd.kernels.stream import NormHint, PreparedRows, UnmergedRows
 
 ABI_VERSION = 1
 _TYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -82,14 +83,20 @@ def _ptr(t: torch.Tensor | None):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
 
-class _UnmergedAttention:
+class _PendingMerge:
     """A decode step's attention output that still lies in the partial results of its key
-    splits: `out` is where the merge would put it."""
+    splits: `out` is where the merge puts it.  Holds the partial results alive."""
 
-    def __init__(self, out, args, partial_o, partial_ml, positions, window):
-        self.out, self.args = out, args                      # args: AttentionMfmaArgs
+    def __init__(self, ops, out, args, partial_o, partial_ml, positions, window):
+        self.ops, self.out, self.args = ops, out, args       # args: AttentionMfmaArgs
         self.partial_o, self.partial_ml = partial_o, partial_ml
         self.positions, self.window = positions, window
+        self.done = False
+
+    def merge(self) -> None:
+        if not self.done:
+            self.ops._call(self.ops.lib.ts_attention_merge, byref(self.args), self.ops._stream())
+            self.done = True
 
 
 class HipOps:
@@ -107,13 +114,14 @@ class HipOps:
             lambda index: torch.cuda.current_stream(index).cuda_stream)
         self._attn_chunk = self.lib.ts_attention_mfma_chunk()
         self._units = torch.cuda.get_device_properties(self.device).multi_processor_count
+        # which kernel takes what: every threshold in one table (kernels/dispatch.py)
+        self.dispatch = default_dispatch()
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
         self._timed_plans = False
         # products of few rows with large weights: ours or the library's, per weight shape
         # (see large_weight_choices)
         self._large_rows, self._large_undecided, self._large_trial = {}, set(), None
-        self._unmerged = None          # an attention output whose merge was deferred
         self.merged_rows = self.lib.ts_gemm_tail_merged_rows()   # rows up to which that pays
         # Above those rows the decode kernel merges its key splits itself: the workgroups of
         # an item count themselves in here and the last one merges.  The kernel leaves every
@@ -137,20 +145,19 @@ class HipOps:
 
     def reset_scratch(self) -> None:
         """Put what this provider keeps between calls back to its start: the arrival counts
-        of the decode kernel's own merge at zero, no deferred merge pending.  Called after a
-        failed call, and by the engine before its warm-up step and before graphs are
-        captured."""
-        self._unmerged = None
+        of the decode kernel's own merge at zero.  Called after a failed call, and by the
+        engine before its warm-up step and before graphs are captured."""
         self._arrivals.zero_()
 
     def _check(self, name, t, dtype=None, shape=None, ndim=None):
         # (written for the case that all is well, which is every call of a working engine:
         # this runs several times before every kernel)
-        if self._unmerged is not None and self._is_unmerged(t):
-            self._merge_now()
         try:
             ok = t.device == self.device and t.is_contiguous()
         except AttributeError:
+            if isinstance(t, UnmergedRows):
+                raise TypeError(f"{name}: an unmerged attention output; this call does not "
+                                "take one (merged() gives the tensor)") from None
             raise TypeError(f"{name}: expected a tensor, got {type(t)}") from None
         if ok and dtype is not None:
             ok = t.dtype is dtype or (dtype.__class__ is tuple and t.dtype in dtype)
@@ -176,21 +183,15 @@ class HipOps:
 
     # ------------------------------------------------------------ deferred merge
     # A decode step's attention whose keys were split over workgroups ends in a merge of the
-    # splits' partial results.  `attend(defer_merge=True)` leaves that merge undone and
-    # remembers it; if the tensor it returned is next handed to `linear_into_stream` (the
-    # output projection in its tail form), that product's kernel merges the rows itself and
-    # a layer has one dependent kernel less.  Any other call of this provider that is given
-    # the tensor runs the merge first, so a caller sees nothing of this as long as the
-    # tensor goes nowhere but into this provider's calls (what `defer_merge` promises).
-    def _is_unmerged(self, t) -> bool:
-        try:
-            return t.data_ptr() == self._unmerged.out.data_ptr()
-        except AttributeError:
-            return False
-
-    def _merge_now(self) -> None:
-        pending, self._unmerged = self._unmerged, None
-        self._call(self.lib.ts_attention_merge, byref(pending.args), self._stream())
+    # splits' partial results.  `attend(defer_merge=True)` may leave that merge undone and
+    # return an `UnmergedRows` handle instead of a tensor; handed to `linear_into_stream`
+    # (the output projection in its tail form), that product's kernel merges the rows itself
+    # and a layer has one dependent kernel less.  The other calls that take activation rows
+    # merge first (`_rows`); nothing else can read the rows by mistake, the handle being no
+    # tensor.
+    @staticmethod
+    def _rows(x):
+        return x.merged() if x.__class__ is UnmergedRows else x
 
     # ------------------------------------------------------------ rows
     def embed(self, table, token_ids):
@@ -211,6 +212,7 @@ class HipOps:
                    token_ids.shape[0], drawn.shape[0], self._stream())
 
     def gather_rows(self, x, rows):
+        x = self._rows(x)
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("rows", rows, torch.int32, ndim=1)
         out = torch.empty(rows.shape[0], x.shape[1], dtype=x.dtype, device=self.device)
@@ -219,6 +221,7 @@ class HipOps:
         return out
 
     def rmsnorm(self, x, weight, eps, out_dtype):
+        x = self._rows(x)
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("norm weight", weight, torch.float32, shape=(x.shape[1],))
         out = torch.empty(x.shape, dtype=out_dtype, device=self.device)
@@ -227,6 +230,7 @@ class HipOps:
         return out
 
     def add_rmsnorm(self, resid, delta, weight, eps, out_dtype):
+        delta = self._rows(delta)
         self._check("resid", resid, torch.float32, ndim=2)
         self._check("delta", delta, self._FLOATS, shape=resid.shape)
         self._check("norm weight", weight, torch.float32, shape=(resid.shape[1],))
@@ -249,6 +253,7 @@ class HipOps:
     # ------------------------------------------------------------ matrix product
     def linear(self, x, weight, out_dtype):
         """x [M, K] times weight [N, K] transposed -> [M, N] in out_dtype."""
+        x = self._rows(x)
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("weight", weight, self._FLOATS, ndim=2)
         M, K = x.shape
@@ -302,39 +307,17 @@ class HipOps:
                    _TYPE_CODE[out_dtype], M, N, K, int(pair), tile, self._stream())
         return out
 
-    # Rows from which a plain bfloat16 product goes to the vendor library (hipBLASLt behind
-    # torch.matmul), as the reference sends every linear layer to its vendor library
-    # (engine/nn/base_layers.py:7-10).  Measured inside captured graphs at the Qwen3-0.6B
-    # shapes: up to 64 rows the weight-streaming kernels here are faster at the layer
-    # products and fuse the norm before (up to 16 rows) and the SwiGLU after; in the wide
-    # layout (a short K) the library is ahead from 17 rows on, and at the output head (a
-    # very large N, where every one of thousands of workgroups reads all rows of x) from 5.
-    # At the layer shapes of the 8B and 32B models (weights above 2^23 elements, products
-    # bound by bandwidth, not latency) every workgroup's reading of the rows of x costs
-    # as much as the weights from 16 rows on, and the library is ahead from 9 rows.
-    # It accumulates in float32 and stores the type asked for: bfloat16 activations, and
-    # float32 logits at the output head (the reference's logits are bfloat16).
-    LIBRARY_ROWS = 65
-    LIBRARY_ROWS_WIDE = 17
-    LIBRARY_ROWS_HEAD = 5
-    HEAD_COLUMNS = 16384
-    LIBRARY_ROWS_LARGE = 9
-    LARGE_WEIGHT = 1 << 23
-
-    # Stacked gate/up weights up to which the product of many rows with the SiLU-multiply
-    # in its epilogue is the LDS-tiled kernel's.  Measured in captured graphs against the
-    # library's product followed by the SiLU-multiply kernel: at the 0.6B shape (2 x 3072
-    # x 1024) 0.56 to 0.87 of their time from 128 to 8192 rows, because the [M, 2 I]
-    # intermediate is neither written nor read; at the 8B shape 0.85 to 1.07 and at the 32B
-    # shape 1.02 to 1.20, the library's product itself being 10 to 20 % ahead of the tiled
-    # kernel's at large sizes.  Plain products stay the library's for the same reason.
-    TILED_PAIR_WEIGHT = 1 << 23
+    # Which rows and sizes go to the vendor library, to the LDS-tiled kernel or stay with
+    # the weight-streaming kernels is `self.dispatch`'s (kernels/dispatch.py: every
+    # threshold with the shapes it was measured on).  The library accumulates in float32
+    # and stores the type asked for: bfloat16 activations, and float32 logits at the output
+    # head (the reference's logits are bfloat16).
 
     def _tiled_pair_ok(self, x, weight, out_dtype):
         M, K = x.shape
         inner = weight.shape[0] // 2
         return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and out_dtype == torch.bfloat16 and weight.numel() <= self.TILED_PAIR_WEIGHT
+                and out_dtype == torch.bfloat16 and weight.numel() <= self.dispatch.tiled_pair_weight
                 and self._library_rows(M, weight.shape[0], K)
                 and self.lib.ts_gemm_tiled_fits(M, inner, K, 1) == 1)
 
@@ -354,7 +337,7 @@ class HipOps:
         models of other shapes in the same process get their own."""
         if not self._large_undecided:
             return ()
-        return (self.LIBRARY_ROWS_LARGE, 1)
+        return (self.dispatch.library_rows_large, 1)
 
     def try_large_weight_rows(self, rows) -> None:
         """For the shapes without a choice: `rows` for now (None: the default again)."""
@@ -369,18 +352,19 @@ class HipOps:
 
     def _library_rows(self, M, N, K):
         """Whether a bfloat16 product of M rows with a weight [N, K] is the library's."""
-        if M >= self.LIBRARY_ROWS:
+        d = self.dispatch
+        if M >= d.library_rows:
             return True
-        if M >= self.LIBRARY_ROWS_HEAD and N >= self.HEAD_COLUMNS:
+        if M >= d.library_rows_head and N >= d.head_columns:
             return True
-        if N * K > self.LARGE_WEIGHT:
+        if N * K > d.large_weight:
             rows = self._large_rows.get((N, K))
             if rows is None:
                 self._large_undecided.add((N, K))
-                rows = self.LIBRARY_ROWS_LARGE if self._large_trial is None else self._large_trial
+                rows = d.library_rows_large if self._large_trial is None else self._large_trial
             if M >= rows:
                 return True
-        return M >= self.LIBRARY_ROWS_WIDE and self.lib.ts_gemm_mfma_layout(N, K) == 2
+        return M >= d.library_rows_wide and self.lib.ts_gemm_mfma_layout(N, K) == 2
 
     @staticmethod
     def _mfma_ok(x, weight):
@@ -399,11 +383,12 @@ class HipOps:
         if hint is None or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 \
                 or hint.weight.dtype != torch.bfloat16:
             return None
-        unmerged = self._unmerged if self._unmerged is not None and self._is_unmerged(x) else None
-        if unmerged is not None:
-            prepared = self._merged_into_stream(unmerged, x, weight, resid, hint)
-            if prepared is not None:
-                return prepared
+        if x.__class__ is UnmergedRows:
+            if not x.is_merged:
+                prepared = self._merged_into_stream(x._pending, x, weight, resid, hint)
+                if prepared is not None:
+                    return prepared
+            x = x.merged()
         self._check("x", x, torch.bfloat16, ndim=2)
         self._check("weight", weight, torch.bfloat16, ndim=2)
         M, K = x.shape
@@ -431,9 +416,8 @@ class HipOps:
         a = unmerged.args.base
         M, K = x.shape
         N = weight.shape[0]
-        if K != a.nq * a.hd or weight.shape[1] != K or M != a.num_tokens \
-                or not x.is_contiguous() or hint.weight.shape[1] != N \
-                or M > self.merged_rows:
+        if len(x.shape) != 2 or K != a.nq * a.hd or weight.shape[1] != K or M != a.num_tokens \
+                or hint.weight.shape[1] != N or M > self.merged_rows:
             return None
         next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
         parts = self.lib.ts_gemm_tail_parts(M, N)
@@ -446,15 +430,12 @@ class HipOps:
         self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
         rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
         sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
-        # (the merge stays pending until the kernel that does it has been launched: a refusal
-        # raises, and a failed call clears it with the rest of the scratch state)
         self._call(self.lib.ts_gemm_tail_merged_bf16, _ptr(unmerged.partial_o),
                    _ptr(unmerged.partial_ml), _ptr(unmerged.positions),
                    unmerged.args.num_splits, a.nq, a.nkv, a.hd,
                    0 if unmerged.window is None else int(unmerged.window), _ptr(weight),
                    _ptr(resid), _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N,
                    self._stream())
-        self._unmerged = None
         return PreparedRows(rows, sumsq, hint)
 
     def _prepared_linear(self, resid, prepared, norm_weight, eps, weight, out_dtype, silu_mul):
@@ -484,6 +465,7 @@ class HipOps:
         if isinstance(delta, PreparedRows):     # already added in, by linear_into_stream
             return self._prepared_linear(resid, delta, norm_weight, eps, weight, out_dtype,
                                          silu_mul)
+        delta = self._rows(delta)
         M, K = resid.shape
         self._check("weight", weight, self._FLOATS, ndim=2)
         if weight.shape[1] != K:
@@ -518,6 +500,7 @@ class HipOps:
 
     def linear_silu_mul(self, x, weight, out_dtype):
         """silu(x Wg^T) * (x Wu^T) for weight = [Wg; Wu] stacked by rows -> [M, N/2]."""
+        x = self._rows(x)
         self._check("x", x, self._FLOATS, ndim=2)
         self._check("weight", weight, self._FLOATS, ndim=2)
         M, K = x.shape
@@ -675,7 +658,9 @@ class HipOps:
         the row then brings `kv_in_row` = `num_kv_heads` key and value heads) and attention
         over the cache -> [T, num_heads, head_dim].  A decode step (one token per entry)
         in bfloat16 is one kernel; anything else is the preparation kernel and
-        paged_attention."""
+        paged_attention.  With `defer_merge` the result may be an `UnmergedRows` handle of
+        that shape instead of a tensor (the caller hands it to `linear_into_stream` or
+        `linear`, or asks it for the tensor with `merged()`)."""
         T = qkv.shape[0]
         fused = (qkv.dtype == torch.bfloat16 and cache.k_pages.dtype == torch.bfloat16
                  and bool(write_cache) == bool(kv_in_row)
@@ -703,16 +688,14 @@ class HipOps:
         d = AttentionDecodeArgs()
         d.qkv, d.q_weight, d.k_weight = qa.qkv, qa.q_weight, qa.k_weight
         d.cos, d.sin, d.eps, d.kv_in_row = qa.cos, qa.sin, eps, kv_in_row
-        if self._unmerged is not None:      # one that nobody took: its tensor is dead
-            self._unmerged = None
-        self._attention_decode(a, batch, num_heads // num_kv_heads, d, out if defer_merge else None,
-                               window)
-        return out
+        pending = self._attention_decode(a, batch, num_heads // num_kv_heads, d,
+                                         out if defer_merge else None, window)
+        return out if pending is None else UnmergedRows(pending, out.shape)
 
     def _attention_decode(self, a, batch, group, d=None, defer_out=None, window=None):
         """One token per entry: workgroups per (entry, key/value head, share of the keys).
-        `defer_out`: the output tensor, if the merge of the splits is to be left undone
-        and remembered (see `_is_unmerged`)."""
+        `defer_out`: the output tensor, if the merge of the splits may be left undone; then
+        the pending merge is returned (else None)."""
         d = d or AttentionDecodeArgs()
         m = d.m
         m.base = a
@@ -735,16 +718,12 @@ class HipOps:
         self._call(self.lib.ts_attention_decode, byref(d), self._stream())
         if d.defer_merge:
             kept = AttentionMfmaArgs.from_buffer_copy(m)
-            self._unmerged = _UnmergedAttention(defer_out, kept, po, pml, batch.positions, window)
-
-    # Workgroups (entries x key/value heads) up to which a decode step takes the decode
-    # kernel; with more, the chip is full anyway and the smaller workgroups of the general
-    # kernel do better.  Measured in captured graphs at 16 query / 8 key heads of 128.
-    DECODE_ITEMS = 512
+            return _PendingMerge(self, defer_out, kept, po, pml, batch.positions, window)
+        return None
 
     def _decode_fits(self, batch, num_kv_heads, group, head_dim, page_size, fused):
         items = batch.num_entries * num_kv_heads * -(-group // 16)
-        return (batch.max_q_len == 1 and items <= self.DECODE_ITEMS
+        return (batch.max_q_len == 1 and items <= self.dispatch.decode_items
                 and self.lib.ts_attention_decode_fits(head_dim, page_size, int(fused)) == 1)
 
     def _decode_splits(self, items, span):
@@ -787,8 +766,10 @@ class HipOps:
         max_chunks = max(1, -(-span // chunk))
         # few tiles (decode): a workgroup per tile and chunk, its waves share the chunk;
         # many tiles (prompts): a wavefront per tile walks its keys
-        cooperative = items <= 1024
-        splits = min(max_chunks, max(1, (512 if cooperative else 4096) // items))
+        d = self.dispatch
+        cooperative = items <= d.cooperative_items
+        splits = min(max_chunks, max(1, (d.cooperative_workgroups if cooperative
+                                         else d.per_wave_workgroups) // items))
         m.cooperative = int(cooperative)
         m.tiles = tiles_dev.data_ptr() if tiles_dev is not None else None
         m.num_tiles = num_tiles
@@ -800,20 +781,14 @@ class HipOps:
         self._call(self.lib.ts_attention_mfma, byref(m), self._stream())
 
     def _prefill_tiles(self, batch, num_kv_heads, group):
-        """Tokens per 16-row tile if the step holds portions of prompts (enough 16-row
-        tiles for the kernel whose waves share key/value blocks through LDS), else None.
-        Measured at 16 query and 8 key/value heads of 128 against the general kernel: one
-        portion of 256 tokens 11.0 against 16.6 us, 1,024 tokens 21.5 against 34.4, 1,536
-        tokens 34.0 against 96.8; below that the two are equal."""
+        """Tokens per 16-row tile if the step goes to the kernel for long portions (enough
+        16-row wave tiles for the kernel whose waves share key/value blocks through LDS;
+        the counts and what they were measured on: kernels/dispatch.py), else None."""
         tokens_per_tile = 16 // min(group, 16)
         tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
         waves = tiles16 * num_kv_heads * -(-group // 16)
-        # a step of single tokens only takes it where the chip is full without splitting keys:
-        # from 1,024 wave tiles (128 entries at 8 key/value heads) it is ahead of the general
-        # kernel at every context length tried (136 entries: 34 against 41 us at 300 tokens
-        # each, 130 against 150 at 100 to 2,000, 426 against 445 at 4,000; 200 entries: 46
-        # / 51, 180 / 223, 608 / 653), at 576 to 768 it is level or behind
-        enough = 256 if batch.max_q_len >= 32 else 1024
+        d = self.dispatch
+        enough = d.portion_tiles if batch.max_q_len >= d.portion_tokens else d.single_token_tiles
         return tokens_per_tile if waves >= enough else None
 
     def _attention_tiles(self, batch, tokens, longest_first=False):

@@ -36,6 +36,43 @@ class PreparedRows:
     hint: NormHint
 
 
+class UnmergedRows:
+    """What `attend(defer_merge=True)` may return in place of a tensor: a decode step's
+    attention output whose key splits have not been merged yet.  It is deliberately no
+    tensor.  The provider's `linear_into_stream` takes it and lets the product's kernel do
+    the merge; its other calls that take activation rows (`linear`, `norm_linear`, ...)
+    merge first; `merged()` gives the tensor to anyone else; and anything that treats it
+    as a tensor fails loudly instead of reading rows that are not there yet.  `view` gives
+    the same pending rows another logical shape."""
+
+    def __init__(self, pending, shape):
+        self._pending, self.shape = pending, torch.Size(shape)
+
+    @property
+    def dtype(self):
+        return self._pending.out.dtype
+
+    @property
+    def device(self):
+        return self._pending.out.device
+
+    @property
+    def is_merged(self) -> bool:
+        return self._pending.done
+
+    def view(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list, torch.Size)):
+            shape = tuple(shape[0])
+        if torch.Size(shape).numel() != self.shape.numel():
+            raise ValueError(f"cannot view rows of shape {tuple(self.shape)} as {tuple(shape)}")
+        return UnmergedRows(self._pending, shape)
+
+    def merged(self) -> torch.Tensor:
+        """The attention output as a tensor; runs the merge if nothing has yet."""
+        self._pending.merge()
+        return self._pending.out.view(self.shape)
+
+
 def fused_rmsnorm_of(norm):
     """(weight, eps) if `norm` says it is a plain RMSNorm that a kernel may fuse into the
     product after it (it has a `fused_rmsnorm()` that returns them), else None."""

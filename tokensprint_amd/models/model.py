@@ -11,10 +11,10 @@ from __future__ import annotations
 import torch
 
 from tokensprint_amd.models.spec import ModelSpec
+import tokensprint_amd.parts  # noqa: F401  (registers the built-in parts)
 from tokensprint_amd.parts.base import (
-    BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, BuildContext, TensorDecl, build_part,
+    BLOCKS, EMBEDDINGS, HEADS, NORMS, POSITIONS, BuildContext, TensorDecl, build_part,
 )
-from tokensprint_amd.parts.ends import Embedding, Head
 
 
 class Model:
@@ -25,18 +25,22 @@ class Model:
         self.spec, self.ctx = spec, ctx
         for name, pspec in spec.positions.items():
             ctx.positions[name] = build_part(POSITIONS, pspec, ctx)
-        self.embedding = Embedding(dict(spec.embedding.params), ctx)
+        self.embedding = build_part(EMBEDDINGS, spec.embedding, ctx)
         self.blocks = []
-        for layer in spec.layers:
+        for i, layer in enumerate(spec.layers):
             if layer.block not in BLOCKS:
                 raise ValueError(f"unknown block kind '{layer.block}'; registered: {sorted(BLOCKS)}")
-            self.blocks.append(BLOCKS[layer.block](
-                build_part(MIXERS, layer.mixer, ctx),
-                build_part(FEED_FORWARDS, layer.feed_forward, ctx),
-                build_part(NORMS, layer.mixer_norm, ctx),
-                build_part(NORMS, layer.ffn_norm, ctx), ctx))
+            kind = BLOCKS[layer.block]
+            unknown = sorted(set(layer.parts) - set(kind.ROLES))
+            if unknown:
+                raise ValueError(f"layer {i}: a '{layer.block}' block has no parts {unknown}; "
+                                 f"its roles are {sorted(kind.ROLES)}")
+            # every part from the registry its role names; the block checks what it needs
+            built = {role: build_part(kind.ROLES[role][0], pspec, ctx)
+                     for role, pspec in layer.parts.items()}
+            self.blocks.append(kind(built, ctx))
         self.final_norm = build_part(NORMS, spec.final_norm, ctx)
-        self.head = Head(dict(spec.head.params), ctx)
+        self.head = build_part(HEADS, spec.head, ctx)
         self.order = spec.order
 
     # ------------------------------------------------------------ weights
@@ -67,8 +71,8 @@ class Model:
 
     # ------------------------------------------------------------ caches
     def cache_needs(self):
-        """Per run: the cache need of its mixer, or None if the run owns no cache."""
-        return [self.blocks[run.layer].mixer.cache_need() if run.cache_of is None else None
+        """Per run: the cache need of its block, or None if the run owns no cache."""
+        return [self.blocks[run.layer].cache_need() if run.cache_of is None else None
                 for run in self.order]
 
     # ------------------------------------------------------------ step

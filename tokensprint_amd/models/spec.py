@@ -19,15 +19,44 @@ class PartSpec:
     params: Mapping[str, Any] = field(default_factory=dict)
 
 
-@dataclass(frozen=True)
 class LayerSpec:
-    """One set of weights: a mixer and a feed-forward, each behind a norm."""
+    """One set of weights: the parts one block is put together from, by role.
 
-    block: str                 # arrangement of the parts, e.g. "pre_norm"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    Which roles there are, which of them a layer may leave out and which registry serves
+    each is the block kind's business (`Block.ROLES`).  The pre-norm block has `mixer`,
+    `feed_forward`, `mixer_norm` and `ffn_norm`, which may also be given in that order;
+    another block kind may name other roles (a norm behind the mixer, no feed-forward).
+    """
+
+    __slots__ = ("block", "parts")
+    _ORDER = ("mixer", "feed_forward", "mixer_norm", "ffn_norm")
+
+    def __init__(self, block: str, *in_order: PartSpec, **by_role: PartSpec | None) -> None:
+        if len(in_order) > len(self._ORDER):
+            raise TypeError(f"at most {len(self._ORDER)} parts can be given by position")
+        parts = dict(zip(self._ORDER, in_order))
+        for role, spec in by_role.items():
+            if role in parts:
+                raise TypeError(f"part '{role}' given twice")
+            if spec is not None:
+                parts[role] = spec
+        object.__setattr__(self, "block", block)
+        object.__setattr__(self, "parts", parts)
+
+    def __setattr__(self, name, value):
+        raise AttributeError("a LayerSpec is not changed after it is made")
+
+    def __getattr__(self, role):
+        try:
+            return self.parts[role]
+        except KeyError:
+            raise AttributeError(f"this layer has no part '{role}'") from None
+
+    def __eq__(self, other):
+        return isinstance(other, LayerSpec) and (self.block, self.parts) == (other.block, other.parts)
+
+    def __repr__(self):
+        return f"LayerSpec({self.block!r}, " + ", ".join(f"{k}={v!r}" for k, v in self.parts.items()) + ")"
 
 
 @dataclass(frozen=True)

@@ -101,8 +101,9 @@ class GroupedQueryAttention(StreamProducts, Mixer):
                 num_kv_heads=self.nkv, kv_in_row=nkv_here, head_dim=self.hd,
                 q_weight=self.w_qnorm, k_weight=self.w_knorm, eps=self.eps,
                 cos_sin=tables, scale=self.scale, window=self.window,
-                # the result goes nowhere but into the output projection, a call of the
-                # same provider, which may then finish attention's last stage itself
+                # the result goes into the output projection, a product of the same provider,
+                # which may then finish attention's last stage itself: it may come back as
+                # a handle (kernels.stream.UnmergedRows) in place of a tensor
                 defer_merge=True)
         else:
             # the encoding has no rotary table: norm only, let it encode, then store

@@ -7,8 +7,8 @@ the step's batch description and, for a mixer, the cache of the run it executes.
 No part knows which model it is in.
 
 Registries map a `kind` string to a class, one registry per role:
-`MIXERS`, `FEED_FORWARDS`, `NORMS`, `POSITIONS`, `BLOCKS`.  A test or a new
-architecture adds a part with `register(MIXERS, "my_kind")(MyClass)`.
+`MIXERS`, `FEED_FORWARDS`, `NORMS`, `POSITIONS`, `BLOCKS`, `EMBEDDINGS`, `HEADS`.  A test
+or a new architecture adds a part with `register(MIXERS, "my_kind")(MyClass)`.
 """
 
 from __future__ import annotations
@@ -164,8 +164,30 @@ class FeedForward(Part):
         return self.forward(h, batch), resid
 
 
+class TokenEmbedding(Part):
+    """The model's first part: token ids (int32 [T]) -> the residual stream, float32
+    [T, width]."""
+
+    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class OutputHead(Part):
+    """The model's last part: rows of the residual stream -> logits, float32 [R, vocab]."""
+
+    def forward_from_stream(self, resid: torch.Tensor, delta, norm: Norm) -> torch.Tensor:
+        """Logits of the rows of the stream (`resid` float32, `delta` the last sub-layer's
+        output not yet added, or None) behind the model's final `norm`."""
+        raise NotImplementedError
+
+
 class Block:
     """Arrangement of one layer's parts around the residual stream.
+
+    `ROLES` names the parts a layer of this kind is made of: role -> (registry, required).
+    The model builds each part a `LayerSpec` gives from the role's registry and hands them
+    over by role; they become attributes of the block (a role the layer leaves out is
+    None).
 
     The stream travels as (resid, delta): resid is float32 [T, width]; delta is
     the last sub-layer's output not yet added (None at the very start), so the
@@ -174,14 +196,26 @@ class Block:
     that hint's protocol defines; only that reader ever sees it.
     """
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 ffn_norm: Norm, ctx: BuildContext) -> None:
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+    ROLES: dict[str, tuple[dict, bool]] = {}
+
+    def __init__(self, parts: dict[str, Part], ctx: BuildContext) -> None:
+        unknown = sorted(set(parts) - set(self.ROLES))
+        missing = sorted(r for r, (_, required) in self.ROLES.items()
+                         if required and parts.get(r) is None)
+        if unknown or missing:
+            raise ValueError(f"{type(self).__name__}: unknown parts {unknown}, missing parts "
+                             f"{missing}; its roles are {sorted(self.ROLES)}")
+        for role in self.ROLES:
+            setattr(self, role, parts.get(role))
         self.ctx = ctx
 
     def parts(self) -> list[Part]:
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward]
+        return [getattr(self, role) for role in self.ROLES if getattr(self, role) is not None]
+
+    def cache_need(self):
+        """What a run of this block keeps per request: its mixer's need, if it has one."""
+        mixer = getattr(self, "mixer", None)
+        return mixer.cache_need() if mixer is not None else None
 
     def entry_hint(self):
         """The `stream_hint` of the part of this block that reads the stream first."""
@@ -199,6 +233,8 @@ FEED_FORWARDS: dict[str, type] = {}
 NORMS: dict[str, type] = {}
 POSITIONS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
+EMBEDDINGS: dict[str, type] = {}
+HEADS: dict[str, type] = {}
 
 
 def register(registry: dict[str, type], kind: str, *, replace: bool = False):

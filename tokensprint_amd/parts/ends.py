@@ -11,10 +11,12 @@ from __future__ import annotations
 import torch
 
 from tokensprint_amd.kernels.stream import fused_rmsnorm_of
-from tokensprint_amd.parts.base import Part, TensorDecl
+from tokensprint_amd.parts.base import (EMBEDDINGS, HEADS, OutputHead, TensorDecl,
+                                        TokenEmbedding, register)
 
 
-class Embedding(Part):
+@register(EMBEDDINGS, "embedding")
+class Embedding(TokenEmbedding):
     """params: weight (checkpoint name), vocab_size."""
 
     def __init__(self, params, ctx):
@@ -36,7 +38,8 @@ class Embedding(Part):
         return []          # a step reads the rows of its tokens, not the table
 
 
-class Head(Part):
+@register(HEADS, "head")
+class Head(OutputHead):
     """params: weight (name), vocab_size, tied (bool: `weight` is the embedding's)."""
 
     def __init__(self, params, ctx):

@@ -10,12 +10,16 @@ engine/models/_api.py:45).
 from __future__ import annotations
 
 import json
+import logging
 from pathlib import Path
 
 import torch
 from safetensors import safe_open
 
 from tokensprint_amd.parts.base import TensorDecl
+
+
+log = logging.getLogger(__name__)
 
 
 class WeightsError(RuntimeError):
@@ -84,18 +88,20 @@ class TensorDict:
         return self._t[name]
 
 
-def held_dtype(decl: TensorDecl, stored: torch.dtype, run_dtype: torch.dtype) -> torch.dtype:
+def held_dtype(decl: TensorDecl, stored: torch.dtype, run_dtype: torch.dtype,
+               cast_32bit: bool = False) -> torch.dtype:
     """The dtype a tensor is held in.
 
     Small vectors are held in float32 (exact for bfloat16 values) and integer
     tables in int32.  Matrices follow the run dtype, except that in a bfloat16 run
-    a matrix the file stores in 32-bit stays 32-bit.
+    a matrix the file stores in 32-bit stays 32-bit (its products then run on the
+    float32 multiply-add kernels) unless `cast_32bit` asks for it to be rounded.
     """
     if decl.role == "table" or not stored.is_floating_point:
         return torch.int32
     if decl.role == "vector" or run_dtype == torch.float32:
         return torch.float32
-    if stored == torch.float32 or stored == torch.float64:
+    if (stored == torch.float32 or stored == torch.float64) and not cast_32bit:
         return torch.float32
     return torch.bfloat16
 
@@ -110,10 +116,12 @@ def check_tensors(decls: dict[str, TensorDecl], source) -> None:
         raise WeightsError(missing, unexpected, wrong)
 
 
-def load_weights(model, source, run_dtype: torch.dtype, device) -> None:
+def load_weights(model, source, run_dtype: torch.dtype, device, cast_32bit: bool = False) -> None:
     """Check `source` against the model's declarations, then hand the tensors over.
 
-    `source` is a model folder path, a `CheckpointFiles` or a `TensorDict`.
+    `source` is a model folder path, a `CheckpointFiles` or a `TensorDict`.  In a bfloat16
+    run matrices stored in 32-bit stay 32-bit, and a warning says how many and what that
+    costs; `cast_32bit` rounds them to bfloat16 instead.
     """
     if isinstance(source, (str, Path)):
         source = CheckpointFiles(source)
@@ -121,9 +129,16 @@ def load_weights(model, source, run_dtype: torch.dtype, device) -> None:
     check_tensors(decls, source)
     have = set(source.names())
     needed = {n for part in model.parts() for n, d in part.tensors().items() if not d.optional}
-    tensors = {}
+    tensors, kept_wide = {}, []
     for name in sorted(needed & have):
         t = source.read(name)
-        tensors[name] = t.to(device=device, dtype=held_dtype(decls[name], t.dtype, run_dtype)
-                             ).contiguous()
+        held = held_dtype(decls[name], t.dtype, run_dtype, cast_32bit)
+        if held == torch.float32 and run_dtype != torch.float32 and decls[name].role == "matrix":
+            kept_wide.append(name)
+        tensors[name] = t.to(device=device, dtype=held).contiguous()
+    if kept_wide:
+        log.warning("%d matrices are stored in 32-bit and stay so in this bfloat16 run (%s, ...): "
+                    "their products run on the float32 multiply-add kernels, many times slower "
+                    "than the bfloat16 ones; load with cast_32bit=True (--cast-weights True) to "
+                    "round them to bfloat16", len(kept_wide), kept_wide[0])
     model.load_tensors(tensors)
