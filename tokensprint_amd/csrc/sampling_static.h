@@ -1,7 +1,6 @@
 // Sampling for callers that cannot allocate device memory: code under HIP graph capture,
 // tight serving loops, harnesses that forbid hipMalloc.  This entry point has no
-// counterpart in the reference (its sampler, engine/generation/sampler.py:5-16, lets
-// torch allocate what it needs); it is here for those callers only.
+// counterpart in the reference; it is here for those callers only.
 //
 // ts_sample_static does what ts_sample does (row r: greedy if temperature[r] <= 1e-10,
 // else a draw from softmax(logits[r] / T) with noise keyed by keys[r]), but the winners
