@@ -824,11 +824,25 @@ def test_paged_attention_finds_one_far_key(ops, gpu_device, dtype):
 @pytest.mark.parametrize("nq,nkv,hd,page,window", [(16, 8, 128, 16, None), (16, 8, 128, 64, 700),
                                                    (8, 8, 96, 16, None), (6, 2, 64, 32, None),
                                                    (40, 2, 32, 16, 300)])
-def test_attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
+@pytest.mark.parametrize("kernel", [2, 0, 3], ids=["default", "turns-of-32", "eight-tiles"])
+def test_attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window, kernel):
     """Portions of prompts long enough for the kernels in which a wavefront walks several
     query tiles: with and without norm weights, rotation, and keys in the row; groups of
     3 and 20 heads, whose 16 rows are not a whole number of tokens (a row past a tile's
-    tokens must not be computed with that tile's key range and stored)."""
+    tokens must not be computed with that tile's key range and stored).  Head sizes 64 and
+    128 have three kernels for this (turns of 64 keys with two sets of waves an item, with
+    eight tiles an item, and turns of 32 keys), chosen by the number of items: each is
+    made to take the same step."""
+    if kernel != 2 and hd not in (64, 128):
+        pytest.skip("one kernel for this head size")
+    ops.lib.ts_attention_prefill_variant(kernel)
+    try:
+        _attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window)
+    finally:
+        ops.lib.ts_attention_prefill_variant(2)
+
+
+def _attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
     dtype = torch.bfloat16
     group = nq // nkv
     per_tile = 16 // min(group, 16)

@@ -551,15 +551,418 @@ __global__ __launch_bounds__(256 * H, H == 1 ? 3 : 2) void attention_prefill_asy
   }
 }
 
+// ---------------------------------------------------------------------------------
+// The walk of the kernel above, 64 keys a turn (two sub-blocks of 32 keys, each laid out in
+// LDS as that kernel lays out a block), with what a turn costs beside its products cut
+// down: one barrier, one wait and one softmax update (row maximum, rescale, row sum) per 64
+// keys instead of two; four independent chains of score products instead of two; and the
+// addresses of a turn's loads formed in a few vector instructions instead of some ninety
+// scalar ones: a lane's address is a 64-bit constant of its own (head, row, slice of the
+// row) plus its page's id times the page stride, one multiply-add per load, the page ids
+// of the turn's four 16-key halves fetched through the scalar cache a turn ahead.
+//
+// A ring of two buffers of 64 keys per set of waves: a turn's loads are sent for right
+// after the barrier that says every wave is through with the buffer they go into (the
+// buffer of the turn before), and are waited for at the start of the next turn.
+//
+// TILES waves share an item's key blocks (an item is TILES consecutive 16-row tiles); H
+// sets of them split the item's turns (set s takes turns s, s + H, ...) and merge through
+// LDS at the end.  `paired` as above.
+// Scores of a 64-key turn for one tile, masked softmax update over all 64, and
+// O^T += V^T P^T for both sub-blocks.  `buf` holds the turn's two sub-blocks (keys, then
+// values, in operand layout).  `between` runs once all the key operands have been asked
+// for (the kernel sends for the next turn's blocks there, while LDS answers).
+//
+// The operands of a stretch of products are asked for together, before the first of them,
+// and the scheduler is told to leave the stretches in that order: the compiler, left
+// alone, asks for an operand only a few instructions before its product, and with two to
+// four waves a SIMD nothing else hides the time LDS takes to answer.  DEEP (kernels that
+// keep two waves a SIMD and so have registers to spare): a stretch is the whole turn, all
+// sixteen key operands before the first score product and all sixteen value operands
+// before the softmax arithmetic.  Otherwise (four waves a SIMD, 128 registers each) the
+// order is the compiler's.
+template <int HD, bool DEEP, typename Between>
+__device__ __forceinline__ void tile_update64(TileState<HD>& t, bf16x8 (*buf)[kWave], int lane, int kb,
+                                              float scale_log2, bool interior, int g,
+                                              Between between) {
+  constexpr int KS = HD / 32, DB = HD / 16, kSlots = 2 * KS + DB;
+  f32x4 st[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) st[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if constexpr (DEEP) {
+    bf16x8 k[4][KS];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int s = 0; s < KS; ++s) k[j][s] = buf[(j / 2) * kSlots + (j % 2) * KS + s][lane];
+    __builtin_amdgcn_sched_barrier(0);
+    between();
+    __builtin_amdgcn_sched_barrier(0);
+    // four chains side by side: a product never waits for the one before it
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        st[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k[j][s], t.q[s], st[j], 0, 0, 0);
+  } else {
+    between();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        st[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[(j / 2) * kSlots + (j % 2) * KS + s][lane],
+                                                        t.q[s], st[j], 0, 0, 0);
+  }
+  bf16x8 v[2][DB];
+  if constexpr (DEEP) {
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) v[sb][db] = buf[sb * kSlots + 2 * KS + db][lane];
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (!interior) {
+    asm volatile("" ::: "memory");   // keeps this a branch
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + (j / 2) * 32 + g * 8 + (j % 2) * 4 + i;
+        st[j][i] = (key <= t.pos && key >= t.lo) ? st[j][i] : -INFINITY;
+      }
+  }
+  float mx = max2(max2(st[0][0], st[0][1]), max2(st[0][2], st[0][3]));
+#pragma unroll
+  for (int j = 1; j < 4; ++j)
+    mx = max2(max2(mx, max2(st[j][0], st[j][1])), max2(st[j][2], st[j][3]));
+  const float m_new = max2(t.m, col4_max(mx) * scale_log2);
+  const float m_use = max2(m_new, -1e30f);
+  const float corr = __builtin_amdgcn_exp2f(t.m - m_use);
+  float ps = 0.f;
+  bf16x8 pv[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[j][i], scale_log2, -m_use));
+      ps += p;
+      pv[j / 2][(j % 2) * 4 + i] = (bf16_t)p;
+    }
+  t.l = t.l * corr + ps;
+  t.m = m_new;
+  if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) t.o[db][i] *= corr;
+  }
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const bf16x8 operand = DEEP ? v[sb][db] : buf[sb * kSlots + 2 * KS + db][lane];
+      t.o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(operand, pv[sb], t.o[db], 0, 0, 0);
+    }
+  }
+}
+
+
+template <int HD, int H, int TILES, int NBUF, bool P16>
+__device__ __forceinline__ void attention_prefill_wide(const AttentionMfmaArgs& args, int paired) {
+  constexpr int KS = HD / 32, DB = HD / 16;
+  constexpr int kSlots = 2 * KS + DB;        // of a sub-block of 32 keys
+  constexpr int L = kSlots / TILES;          // loads a wave sends for per sub-block
+  static_assert(HD % 64 == 0 && kSlots % TILES == 0, "head sizes in steps of 64");
+  constexpr int kBuf = 2 * kSlots;           // slots of a ring buffer: 64 keys
+  constexpr int kAhead = NBUF - 1;           // turns whose blocks are on their way
+  extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
+  typedef bf16x8 (*Slots)[kWave];
+  const AttentionArgs& a = args.base;
+  const int wave_all = uniform(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+  const int wave = wave_all % TILES;             // which of the item's tiles
+  const int set = H == 1 ? 0 : wave_all / TILES; // which of every H turns
+  const Slots ring = (Slots)prefill_lds + set * NBUF * kBuf;
+  const int r = lane % 16, g = lane / 16;
+  const int group = a.nq / a.nkv;
+  const int heads = a.nkv * args.head_blocks;
+  const int head_slot = blockIdx.x % heads;                   // one head per XCD's L2
+  const int rank = blockIdx.x / heads;
+  const int kvh = head_slot / args.head_blocks;
+  const int hb = head_slot % args.head_blocks;
+  const int P = a.page_size, lp = __builtin_ctz(P);
+  const int tq = 16 / args.rows_per_token;
+  const float scale_log2 = a.scale * 1.44269504088896341f;
+
+  // What this lane names in each of its loads of a sub-block: a 64-bit address that lacks
+  // only the page (page id times the page stride, the same for keys and values) and, with
+  // pages above 16 keys, the 16-key half's place inside its page.  Slot q of a sub-block is
+  // a key slot (product q / KS, elements g*8*KS + (q % KS)*8 .. + 7 of the key in row r)
+  // below 2 KS, else the value slot of head elements (q - 2 KS)*16 .. + 15 (this lane's row
+  // r of them, keys g*8 .. + 7).  A lane's keys lie in the sub-block's second half from row
+  // 8 (keys) or from lane group 2 (values).
+  const unsigned page_stride = 2u * (unsigned)a.nkv * P * HD;   // bytes
+  const char* k_head = (const char*)a.k_pages + (int64_t)kvh * P * HD * 2;
+  const char* v_head = (const char*)a.v_pages + (int64_t)kvh * HD * P * 2;
+  const char* cbase[L];
+  bool second[L];
+  unsigned in_bytes[L];                      // bytes per key of the place inside a page
+#pragma unroll
+  for (int i = 0; i < L; ++i) {
+    const int q = wave + TILES * i;
+    if (q < 2 * KS) {
+      const int b = q / KS, s0 = q % KS;
+      const int key16 = ((r / 4) * 8 + b * 4 + r % 4) % 16;
+      cbase[i] = k_head + 2 * (key16 * HD + g * 8 * KS + s0 * 8);
+      second[i] = r >= 8;
+      in_bytes[i] = 2u * HD;
+    } else {
+      cbase[i] = v_head + 2 * (((q - 2 * KS) * 16 + r) * P + (g % 2) * 8);
+      second[i] = g >= 2;
+      in_bytes[i] = 2u;
+    }
+  }
+
+  // The workgroup's items (one, or with `paired` the one at its rank from the front of the
+  // sorted list and the one at the same rank from the back), their first positions and this
+  // lane's query rows: all asked for now, so that the second item begins without the chain
+  // of trips to memory that the first one waits through.
+  int item_of[2], entry_of[2], tok0_of[2], ntok_of[2], pos_of[2];
+  bool has[2] = {true, false};
+  if (paired) {
+    item_of[0] = rank;
+    item_of[1] = args.num_tiles - 1 - rank;
+    has[1] = item_of[1] > rank;
+  } else {
+    const int front = (args.num_tiles + 1) / 2;
+    item_of[0] = rank < front ? rank : args.num_tiles - 1 - (rank - front);
+    item_of[1] = item_of[0];
+  }
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    entry_of[p] = args.tiles[item_of[p] * 3];
+    tok0_of[p] = args.tiles[item_of[p] * 3 + 1];
+    ntok_of[p] = args.tiles[item_of[p] * 3 + 2];
+  }
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    entry_of[p] = uniform(entry_of[p]); tok0_of[p] = uniform(tok0_of[p]); ntok_of[p] = uniform(ntok_of[p]);
+    pos_of[p] = a.positions[tok0_of[p]];
+  }
+  const int hh = hb * 16 + r % args.rows_per_token;
+  const int head = kvh * group + min(hh, group - 1);
+  const int ti = wave * tq + r / args.rows_per_token;
+  bf16x8 q_of[2][KS];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    pos_of[p] = uniform(pos_of[p]);
+    const bool row_ok = r / args.rows_per_token < tq && ti < ntok_of[p] && hh < group;
+    const bf16_t* qrow = (const bf16_t*)a.q +
+                         ((int64_t)(tok0_of[p] + min(ti, ntok_of[p] - 1)) * a.nq + head) * HD;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int s0 = 0; s0 < KS; ++s0)
+      q_of[p][s0] = row_ok && p == 0 ? *(const bf16x8*)(qrow + g * 8 * KS + s0 * 8) : zero8;
+  }
+
+#pragma unroll
+  for (int part = 0; part < 2; ++part) {
+    if (!has[part]) break;
+    const int entry = entry_of[part], tok0 = tok0_of[part], ntok = ntok_of[part];
+    const ConstTable table = (ConstTable)(a.table + (int64_t)entry * a.table_width);
+    const bool row_ok = r / args.rows_per_token < tq && ti < ntok && hh < group;
+    const int pos_first = pos_of[part];
+    const int pos_last = pos_first + ntok - 1;
+    const int lo_all = (a.window > 0) ? max(0, pos_first - a.window + 1) : 0;
+
+    TileState<HD> t;
+    t.pos = row_ok ? pos_first + ti : -1;
+    t.lo = (a.window > 0) ? max(0, t.pos - a.window + 1) : 0;
+    const int tile_first = pos_first + wave * tq;
+    const int tile_last = wave * tq < ntok ? pos_first + min(ntok, (wave + 1) * tq) - 1 : -1;
+    const int tile_lo = (a.window > 0) ? max(0, tile_first - a.window + 1) : 0;
+    const int tile_lo_last = (a.window > 0) ? max(0, tile_last - a.window + 1) : 0;
+    if (part == 0) {
+#pragma unroll
+      for (int s0 = 0; s0 < KS; ++s0) t.q[s0] = q_of[0][s0];
+    } else {
+      const bf16_t* qrow = (const bf16_t*)a.q + ((int64_t)(tok0 + min(ti, ntok - 1)) * a.nq + head) * HD;
+      const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int s0 = 0; s0 < KS; ++s0)
+        t.q[s0] = row_ok ? *(const bf16x8*)(qrow + g * 8 * KS + s0 * 8) : zero8;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) t.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    t.m = -INFINITY;
+    t.l = 0.f;
+
+    // The item's turns of 64 keys, numbered from its first; this set takes turns set,
+    // set + H, ...: `mine` of them, numbered j here.  Every set passes the same number of
+    // barriers.
+    const int key_begin = lo_all & ~63;
+    const int nturns = ((pos_last - key_begin) >> 6) + 1;
+    const int rounds = (nturns + H - 1) / H;
+    const int mine = (nturns - set + H - 1) / H;
+    const int kb_first = key_begin + 64 * set;
+    const int last_page = pos_last >> lp;              // the last page the item may name
+    // page ids of the four 16-key halves of the turn that will be sent for next (a page
+    // beyond the item's last is the last again: its keys are masked; a page that a window
+    // has let go reads page 0, masked as well).  Raw here: what is done with them waits for
+    // the scalar loads, so it is done where they are used, a turn later.
+    int nx[4];
+    typedef int Ids4 __attribute__((ext_vector_type(4), aligned(4)));
+    auto fetch_ids = [&](int kb) {
+      const int i0 = kb >> lp;
+      if (P16 && i0 + 3 <= last_page) {        // four consecutive pages: one scalar load
+        const Ids4 ids = *(const Ids4 __attribute__((address_space(4)))*)(table + i0);
+        nx[0] = ids[0]; nx[1] = ids[1]; nx[2] = ids[2]; nx[3] = ids[3];
+      } else {
+#pragma unroll
+        for (int h = 0; h < 4; ++h) nx[h] = table[min((kb + 16 * h) >> lp, last_page)];
+      }
+    };
+    fetch_ids(kb_first);
+
+    auto issue = [&](int j, int to) {
+      const int kb = kb_first + 64 * H * j;
+      const Slots dst = ring + to * kBuf;
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        const unsigned pa = max(nx[2 * sb], 0), pb = max(nx[2 * sb + 1], 0);
+        const unsigned ia = (kb + 32 * sb) & (P - 1), ib = (kb + 32 * sb + 16) & (P - 1);
+#pragma unroll
+        for (int i = 0; i < L; ++i) {
+          const unsigned page = second[i] ? pb : pa;
+          const char* src = cbase[i] + (uint64_t)page * page_stride;
+          if (!P16) src += (uint64_t)(second[i] ? ib : ia) * in_bytes[i];
+          lds_dma16(src, &dst[sb * kSlots + wave + TILES * i][0]);
+        }
+      }
+      fetch_ids(kb + 64 * H);
+    };
+
+    auto turn = [&](int j, int from, int to) {
+      const int kb = kb_first + 64 * H * j;
+      // this wave's share of turn j has arrived: at most the turn after it is in flight
+      if (kAhead == 2 && j + 1 < mine) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * L));
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();      // every wave's share has, and every wave is through with turn j - 1
+      asm volatile("" ::: "memory");
+      // (the blocks of the turn `kAhead` on are sent for, into the buffer of the turn before
+      // this one, after this turn's key operands have been asked for, so that LDS answers
+      // meanwhile)
+      auto send = [&]() { if (j + kAhead < mine) issue(j + kAhead, to); };
+      if (j < mine && kb <= tile_last && kb + 63 >= tile_lo)
+        tile_update64<HD, true>(t, ring + from * kBuf, lane, kb, scale_log2,
+                                kb + 63 <= tile_first && kb >= tile_lo_last, g, send);
+      else
+        send();
+    };
+
+    // The query rows (both items') are waited for here, once (the empty statement uses
+    // them), and not at their first use inside the loop, where the wait would be for every
+    // block in flight as well; with them gone the vector memory counter counts the blocks'
+    // loads alone.
+#pragma unroll
+    for (int s0 = 0; s0 < KS; ++s0) asm volatile("" : "+v"(t.q[s0]));
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (mine > 0) issue(0, 0);
+    if (kAhead == 2 && mine > 1) issue(1, 1);
+    // written out once per ring buffer so that every turn's buffers are constants
+    if constexpr (NBUF == 2) {
+      for (int j = 0; j < rounds; j += 2) {
+        turn(j, 0, 1);
+        if (j + 1 < rounds) turn(j + 1, 1, 0);
+      }
+    } else {
+      for (int j = 0; j < rounds; j += 3) {
+        turn(j, 0, 2);
+        if (j + 1 < rounds) turn(j + 1, 1, 0);
+        if (j + 2 < rounds) turn(j + 2, 2, 1);
+      }
+    }
+
+    if constexpr (H == 2) {
+      // The second set hands its partial result over in LDS, in the rings' space: values
+      // [tile][element][lane], then the row statistics.
+      float* lds_o = (float*)prefill_lds;
+      float* lds_ml = lds_o + TILES * DB * 4 * kWave;
+      static_assert(H * NBUF * kBuf * kWave * 16 >= (TILES * DB * 4 + TILES * 2) * kWave * 4, "merge area");
+      __syncthreads();                             // the rings have been read for the last time
+      if (set == 1) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) lds_o[((wave * DB + db) * 4 + i) * kWave + lane] = t.o[db][i];
+        lds_ml[(wave * 2) * kWave + lane] = t.m;
+        lds_ml[(wave * 2 + 1) * kWave + lane] = t.l;
+      }
+      __syncthreads();
+      if (set == 0) {
+        const float m1 = lds_ml[(wave * 2) * kWave + lane], l1 = lds_ml[(wave * 2 + 1) * kWave + lane];
+        const float m_use = max2(max2(t.m, m1), -1e30f);
+        const float w0 = __builtin_amdgcn_exp2f(t.m - m_use), w1 = __builtin_amdgcn_exp2f(m1 - m_use);
+        t.l = t.l * w0 + l1 * w1;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float o1 = lds_o[((wave * DB + db) * 4 + i) * kWave + lane];
+            t.o[db][i] = t.o[db][i] * w0 + (w1 == 0.f ? 0.f : o1 * w1);
+          }
+        const float sum = row_sum<HD>(t);
+        if (row_ok)
+          store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+      }
+    } else {
+      const float sum = row_sum<HD>(t);
+      if (row_ok)
+        store_tile<HD>(t, sum, (bf16_t*)a.out + ((int64_t)(tok0 + ti) * a.nq + head) * HD, g);
+    }
+    __syncthreads();       // before the next item's blocks are sent for into these buffers
+  }
+}
+
+// Two waves a SIMD in every form, so a wave may take half the register file.  Four tiles
+// an item: one workgroup of two sets beside rings of two buffers (128 KB).  Eight tiles:
+// one workgroup of eight waves a unit beside a ring of three buffers (96 KB), two turns'
+// blocks on their way, every block it brings in serving eight tiles.
+template <int HD, bool P16>
+__global__ __launch_bounds__(kWave * 8) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attention_prefill_wide_kernel4(AttentionMfmaArgs args, int paired) {
+  attention_prefill_wide<HD, 2, 4, 2, P16>(args, paired);
+}
+template <int HD, bool P16>
+__global__ __launch_bounds__(kWave * 8) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attention_prefill_wide_kernel8(AttentionMfmaArgs args, int paired) {
+  attention_prefill_wide<HD, 1, 8, 3, P16>(args, paired);
+}
+
 // Query tiles per wavefront: as many as the register file holds accumulators for.
 constexpr int tiles_per_wave(int hd) { return hd <= 32 ? 4 : (hd <= 64 ? 2 : 1); }
 
-// Tokens one work item covers, in 16-row tiles: four (one per wave) for the LDS kernel.
-extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size) {
-  return page_size >= 16 && (page_size & (page_size - 1)) == 0 ? 4 : tiles_per_wave(head_dim);
+static int compute_units();
+// Which kernel takes the long portions of head sizes 64 and 128.  2 (the default): turns of
+// 64 keys for few items (two sets of waves per item) and for many (eight tiles an item),
+// turns of 32 keys between; 1: for few items only; 0: turns of 32 keys everywhere; 3: eight
+// tiles an item whatever the number of items (so that tests reach that kernel at small sizes).
+static int g_prefill_variant = 2;
+extern "C" void ts_attention_prefill_variant(int v) { g_prefill_variant = v; }
+
+// Tokens one work item covers, in 16-row tiles, for a step of `tiles16` such tiles over
+// `heads` key/value heads (x blocks of 16 query heads): one tile per wave of the kernels
+// that share key blocks through LDS, i.e. four, or eight where four would give more than
+// two items a compute unit (then eight waves share every block they bring in, and twice
+// the waves fit beside the same rings); the register-only kernel's own count otherwise.
+extern "C" int ts_attention_prefill_tiles(int head_dim, int page_size, int tiles16, int heads) {
+  if (!(page_size >= 16 && (page_size & (page_size - 1)) == 0)) return tiles_per_wave(head_dim);
+  const bool wide = g_prefill_variant >= 2 && head_dim % 64 == 0 && head_dim <= 128;
+  const int64_t items4 = (int64_t)((tiles16 + 3) / 4) * heads;
+  return wide && (g_prefill_variant == 3 || items4 >= 6 * compute_units()) ? 8 : 4;
 }
 
-static int compute_units() {
+int compute_units() {
   static int cus = 0;       // of the device current when first asked; a host's GPUs are alike
   if (cus == 0) {
     int dev = 0, n = 0;
@@ -588,10 +991,39 @@ static int launch_prefill_async(const AttentionMfmaArgs& args, int paired, hipSt
   return 0;
 }
 
+// TILES 4: two sets of four waves per item (`paired` as above).  TILES 8: eight waves.
+template <int HD, int TILES>
+static int launch_prefill_wide(const AttentionMfmaArgs& args, int paired, hipStream_t stream) {
+  const int heads = args.base.nkv * args.head_blocks;
+  const dim3 grid((paired ? (args.num_tiles + 1) / 2 : args.num_tiles) * heads);
+  const size_t lds = (size_t)(TILES == 8 ? 3 : 4) * 2 * (2 * (HD / 32) + HD / 16) * kWave * 16;
+  const bool p16 = args.base.page_size == 16;
+  void (*kernel)(AttentionMfmaArgs, int);
+  if constexpr (TILES == 8)
+    kernel = p16 ? attention_prefill_wide_kernel8<HD, true> : attention_prefill_wide_kernel8<HD, false>;
+  else
+    kernel = p16 ? attention_prefill_wide_kernel4<HD, true> : attention_prefill_wide_kernel4<HD, false>;
+  static bool raised[2] = {false, false};     // per instantiation
+  if (!raised[p16]) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      TS_FAIL("attention_prefill: cannot raise the LDS limit to %zu bytes", lds);
+    raised[p16] = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kWave * 8), lds, stream, args, paired);
+  return 0;
+}
+
 template <int HD>
 static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream) {
-  if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
   const int items = args.num_tiles * args.base.nkv * args.head_blocks;
+  if constexpr (HD % 64 == 0 && HD <= 128) {
+    if (args.tiles_per_wave == 8) {
+      if (g_prefill_variant < 1) TS_FAIL("attention_prefill: items of 8 tiles need the 64-key kernel");
+      return launch_prefill_wide<HD, 8>(args, 0, stream);
+    }
+  }
+  if (args.tiles_per_wave != 4) TS_FAIL("attention_prefill: the LDS kernel takes items of 4 tiles");
   if constexpr (HD % 64 == 0 && HD <= 128) {
     // Up to two items a compute unit: two sets of waves per item, and the items paired (a
     // long one and a short one per workgroup) once there are more items than units, so
@@ -601,6 +1033,8 @@ static int launch_prefill_lds(const AttentionMfmaArgs& args, hipStream_t stream)
     // paired, 35.7 unpaired; 2,048 tokens 42.6 paired, 48.8 with one set; 2,560 tokens 63.9
     // with one set, 92.7 with two sets paired, which then need a second round.)
     const int units = compute_units();
+    if (g_prefill_variant >= 1 && items <= 2 * units)
+      return launch_prefill_wide<HD, 4>(args, items > units, stream);
     if (items <= 2 * units) return launch_prefill_async<HD, 2>(args, items > units, stream);
     return launch_prefill_async<HD, 1>(args, 0, stream);
   } else {

@@ -748,7 +748,9 @@ class HipOps:
         m.rows_per_token, m.head_blocks = rows_per_token, head_blocks
         # long portions of prompts: a wavefront takes several query tiles and walks alone
         if self._prefill_tiles(batch, a.nkv, group) is not None:
-            tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size)
+            tiles16 = sum(-(-n // tokens_per_tile) for n in batch.q_lens)
+            tpw = self.lib.ts_attention_prefill_tiles(a.hd, a.page_size, tiles16,
+                                                      a.nkv * head_blocks)
             tiles_dev, num_tiles = self._attention_tiles(batch, tokens_per_tile * tpw,
                                                          longest_first=True)
             m.tiles, m.num_tiles, m.tiles_per_wave = tiles_dev.data_ptr(), num_tiles, tpw
