@@ -1,8 +1,10 @@
 // C[M,N] = A[M,K] * W[N,K]^T with float32 fused multiply-adds only: no matrix-core
 // instruction and no reduced-precision mode, whatever the operand types.  This is the
 // product of the float32 path and of any bfloat16 run whose weights are held in 32-bit.
-// Every output element adds its K products in index order with one accumulator, so its
-// value does not depend on M or on which other rows are in the call.
+// Every output element adds its K products in an order fixed by K alone (per lane in
+// index order and then across the lanes of a wavefront; in index order with one
+// accumulator in the tiled kernel, which serves a K that is no multiple of 4), so its value
+// does not depend on which other rows are in the call.
 #include "common.h"
 
 constexpr int kTile = 64;   // output tile edge per workgroup
@@ -54,11 +56,14 @@ __global__ __launch_bounds__(256) void gemm_fma_kernel(const TA* __restrict__ A,
   }
 }
 
-// Up to 16 rows of A (decode steps): a thread per output column and one workgroup of 64
-// threads per 64 columns, so the columns spread over the chip.  A thread walks its row of
-// W in 16-byte pieces (the lines it touches stay in the first-level cache until it has
-// used them up), the rows of A come through scalar loads, the same for every thread.
-// The products of an output element are added in index order, as in the tiled kernel.
+// The kernel for every K that is a multiple of 4: a wavefront per four output columns and
+// up to 16 rows of A, so that a row of W is read by 64 lanes side by side (a kilobyte a load
+// instruction) and a decode step's columns spread over the chip.  Lane l takes elements
+// 4 l .. 4 l + 3 of every stretch of 256 of K, adds its products in index order, and the 64
+// lanes' sums are added in a fixed butterfly: the order depends on K alone, never on M or
+// on which other rows are in the call, so a row's result is the same to the bit however
+// the rows are batched (more than 16 rows are further workgroups along y).  The rows of A
+// are the same for every wavefront and come out of the caches.
 typedef __attribute__((ext_vector_type(4))) float f32x4_fma;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_fma;
 __device__ __forceinline__ f32x4_fma load4_fma(const float* p) { return *(const f32x4_fma*)p; }
@@ -67,47 +72,61 @@ __device__ __forceinline__ f32x4_fma load4_fma(const bf16_t* p) {
   return f32x4_fma{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
 }
 
+constexpr int kColumnsPerWave = 4;
+
 template <typename TA, typename TW, typename TC, int MR>
-__global__ __launch_bounds__(64) void gemm_fma_rows_kernel(const TA* __restrict__ A,
-                                                           const TW* __restrict__ W,
-                                                           TC* __restrict__ C, int M, int N, int K) {
-  const int64_t n = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  const TW* wrow = W + min(n, (int64_t)N - 1) * K;
-  float acc[MR];
+__global__ __launch_bounds__(256) void gemm_fma_rows_kernel(const TA* __restrict__ A,
+                                                            const TW* __restrict__ W,
+                                                            TC* __restrict__ C, int M, int N, int K) {
+  constexpr int CPW = kColumnsPerWave;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * CPW;
+  if (n0 >= N) return;
+  const int m0 = blockIdx.y * MR;
+  A += (int64_t)m0 * K;
+  C += (int64_t)m0 * N;
+  M -= m0;
+  float acc[MR][CPW];
 #pragma unroll
-  for (int m = 0; m < MR; ++m) acc[m] = 0.f;
-  const int k4 = K / 4 * 4;
-  int k = 0;
-  for (; k < k4; k += 4) {
-    const f32x4_fma w = load4_fma(wrow + k);
+  for (int m = 0; m < MR; ++m)
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) acc[m][c] = 0.f;
+  for (int k = lane * 4; k < K; k += kWave * 4) {
+    f32x4_fma w[CPW];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) w[c] = load4_fma(W + min(n0 + c, (int64_t)N - 1) * K + k);
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
       const f32x4_fma a = load4_fma(A + (int64_t)min(m, M - 1) * K + k);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[m] = fmaf(a[e], w[e], acc[m]);
+      for (int c = 0; c < CPW; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[m][c] = fmaf(a[e], w[c][e], acc[m][c]);
     }
   }
-  for (; k < K; ++k) {
-    const float w = to_f32(wrow[k]);
-#pragma unroll
-    for (int m = 0; m < MR; ++m)
-      acc[m] = fmaf(to_f32(A[(int64_t)min(m, M - 1) * K + k]), w, acc[m]);
-  }
-  if (n >= N) return;
 #pragma unroll
   for (int m = 0; m < MR; ++m)
-    if (m < M) C[(int64_t)m * N + n] = from_f32<TC>(acc[m]);
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      float v = acc[m][c];
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+      if (lane == 0 && m < M && n0 + c < N) C[(int64_t)m * N + n0 + c] = from_f32<TC>(v);
+    }
 }
 
 template <typename TA, typename TW, typename TC>
 static void launch_rows(const TA* A, const TW* W, TC* C, int M, int N, int K, hipStream_t stream) {
-  const dim3 grid((N + 63) / 64);
+  const int columns = (N + 4 * kColumnsPerWave - 1) / (4 * kColumnsPerWave);
+  const dim3 grid(columns, M <= 16 ? 1 : (M + 15) / 16);
   if (M == 1)
-    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 1>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 1>), grid, dim3(256), 0, stream, A, W, C, M, N, K);
   else if (M <= 4)
-    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 4>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 4>), grid, dim3(256), 0, stream, A, W, C, M, N, K);
+  else if (M <= 8)
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 8>), grid, dim3(256), 0, stream, A, W, C, M, N, K);
   else
-    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 16>), grid, dim3(64), 0, stream, A, W, C, M, N, K);
+    hipLaunchKernelGGL((gemm_fma_rows_kernel<TA, TW, TC, 16>), grid, dim3(256), 0, stream, A, W, C, M, N, K);
 }
 
 extern "C" int ts_gemm_fma(const void* a, int a_type, const void* w, int w_type, void* c,
@@ -115,7 +134,9 @@ extern "C" int ts_gemm_fma(const void* a, int a_type, const void* w, int w_type,
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) TS_FAIL("gemm: K=%d", K);
   // rows of 4 elements must start on 16 (float32) or 8 (bfloat16) bytes for the row kernel
-  const bool rows_ok = M <= 16 && K % 4 == 0 && (((uintptr_t)a | (uintptr_t)w) & 15) == 0;
+  // (a property of K and of the buffers, not of M: which kernel serves a weight never
+  // depends on the number of rows)
+  const bool rows_ok = K % 4 == 0 && (((uintptr_t)a | (uintptr_t)w) & 15) == 0 && (M + 15) / 16 <= 65535;
   if (rows_ok) {
     TS_DISPATCH_TYPE(a_type, TA, TS_DISPATCH_TYPE(w_type, TW, TS_DISPATCH_TYPE(c_type, TC,
         launch_rows<TA, TW, TC>((const TA*)a, (const TW*)w, (TC*)c, M, N, K, stream))));
