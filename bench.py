@@ -287,6 +287,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--model", default="qwen3-0.6b")
     ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--context", type=int, default=4096,
+                    help="the benchmark's context length: the long-context points decode at "
+                         "half of it and at it")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode run")
     ap.add_argument("--skip-fp32", action="store_true", help="no float32 decode point")
     ap.add_argument("--only-prefill", action="store_true",
@@ -302,7 +305,7 @@ def main() -> int:
     raw = load_named_config(args.model)
     full_layers = raw["num_hidden_layers"]
     layers = args.layers or full_layers
-    ctx_len, page = 4096, 16
+    ctx_len, page = args.context, 16
     dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
     item = 2 if dt_name == "bf16" else 4
     vocab = raw["vocab_size"]
