@@ -877,6 +877,46 @@ def _attend_long_portions(ops, gpu_device, nq, nkv, hd, page, window):
         torch.testing.assert_close(out.float(), ref.float(), **tol(dtype))
 
 
+@pytest.mark.parametrize("page", [16, 64])
+@pytest.mark.parametrize("kernel", [2, 0, 3], ids=["default", "turns-of-32", "eight-tiles"])
+def test_long_portion_finds_one_far_key(ops, gpu_device, kernel, page):
+    """Random keys would hide a block that a kernel for long portions skips, reads from the
+    wrong page or masks by mistake: among two thousand keys one more changes a bfloat16
+    result by less than the tolerance.  Here one key at a time, at the edges of pages, of
+    32-key sub-blocks, of 64-key turns and of the sets' alternating turns, is made to
+    dominate every later query's scores: rows from that position on must return its value
+    row, rows before it must not."""
+    dtype = torch.bfloat16
+    nq, nkv, hd, S = 16, 8, 128, 1100          # 1100 tokens: 552 tiles of 16 rows, 4,416 wave tiles
+    batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
+                                            spans=[(0, S)], seed=31)
+    assert ops._prefill_tiles(batch, nkv, nq // nkv) is not None
+    q = rand((S, nq, hd), dtype, gpu_device, 32)
+    direction = rand((hd,), torch.float32, gpu_device, 33)
+    direction = direction / direction.norm()
+    # every query gets a large component along one direction; a key that is 6 x that
+    # direction scores about 6 * 8 above the rest (scale 1)
+    q = (q.float() * 0.2 + 8.0 * direction).to(dtype)
+    ops.lib.ts_attention_prefill_variant(kernel)
+    try:
+        for far in (0, 15, 16, 31, 32, 63, 64, 65, 127, 128, 191, 192, 511, 512, 1023, 1024, 1087, 1099):
+            k_pages = cache.k_pages.clone()
+            phys = int(table[0, far // page])
+            k_pages[phys, :, far % page] = (6.0 * direction).to(dtype)
+            mine = type(cache)(cache.group, cache.page_size, cache.num_pages, k_pages, cache.v_pages)
+            out = ops.paged_attention(q, batch, table, mine, num_heads=nq, num_kv_heads=nkv,
+                                      head_dim=hd, scale=1.0, window=None).float()
+            want = cache.v_pages[phys, :, :, far % page].float()           # [nkv, hd]
+            want = want.repeat_interleave(nq // nkv, dim=0)                # [nq, hd]
+            later = out[far:]                                               # rows that see the key
+            assert (later - want).abs().max() < 3e-2, f"key {far}: {(later - want).abs().max():.3f}"
+            if far:
+                earlier = out[:far]
+                assert (earlier - want).abs().max() > 0.3, f"key {far} shows to rows before it"
+    finally:
+        ops.lib.ts_attention_prefill_variant(2)
+
+
 @pytest.mark.parametrize("ctx", [700, 2500])
 def test_attend_finds_one_far_key_in_a_decode_step(ops, gpu_device, ctx):
     """The same through the fused decode call (no norm, no rotation, so the query is the
