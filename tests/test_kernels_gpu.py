@@ -529,22 +529,32 @@ def test_paged_attention_long_portions(ops, gpu_device, nq, nkv, hd, page, windo
 
 
 @pytest.mark.parametrize("window", [40, 100, 333])
-def test_long_portions_under_a_window_come_out_the_same_every_time(ops, gpu_device, window):
+@pytest.mark.parametrize("spans,kernel", [
+    ([(0, 1212), (333, 1), (50, 1027), (700, 700)], 2),     # many items: turns of 32 keys
+    ([(0, 700), (333, 1), (50, 500), (700, 300)], 2),       # few items: turns of 64, two sets
+    ([(0, 1212), (333, 1), (50, 1027), (700, 700)], 3),     # turns of 64, eight tiles an item
+], ids=["turns-of-32", "two-sets", "eight-tiles"])
+def test_long_portions_under_a_window_come_out_the_same_every_time(ops, gpu_device, window, spans,
+                                                                   kernel):
     """Under a window the waves of a workgroup have different blocks to skip, so some run a
     turn ahead of the others; a block sent for into a buffer that a slower wave still reads
-    would show as a result that differs from launch to launch."""
+    would show as a result that differs from launch to launch.  Each of the three kernels
+    for long portions of this head size."""
     dtype, nq, nkv, hd, page = torch.bfloat16, 16, 8, 128, 16
-    spans = [(0, 1212), (333, 1), (50, 1027), (700, 700)]
     batch, cache, table, _ = paged_scenario(gpu_device, dtype, nkv=nkv, hd=hd, page_size=page,
                                             spans=spans, seed=35)
     assert ops._prefill_tiles(batch, nkv, nq // nkv) is not None
     q = rand((batch.num_tokens, nq, hd), dtype, gpu_device, 36)
     kw = dict(num_heads=nq, num_kv_heads=nkv, head_dim=hd, scale=hd ** -0.5, window=window)
-    first = ops.paged_attention(q, batch, table, cache, **kw).clone()
-    ref = REF.paged_attention(q, batch, table, cache, **kw)
-    torch.testing.assert_close(first.float(), ref.float(), **tol(dtype))
-    for _ in range(30):
-        assert torch.equal(ops.paged_attention(q, batch, table, cache, **kw), first)
+    ops.lib.ts_attention_prefill_variant(kernel)
+    try:
+        first = ops.paged_attention(q, batch, table, cache, **kw).clone()
+        ref = REF.paged_attention(q, batch, table, cache, **kw)
+        torch.testing.assert_close(first.float(), ref.float(), **tol(dtype))
+        for _ in range(30):
+            assert torch.equal(ops.paged_attention(q, batch, table, cache, **kw), first)
+    finally:
+        ops.lib.ts_attention_prefill_variant(2)
 
 
 DECODE_SPANS = [(0, 1), (1, 1), (31, 1), (32, 1), (127, 1), (128, 1), (129, 1), (255, 1),
