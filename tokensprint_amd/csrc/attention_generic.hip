@@ -10,6 +10,16 @@
 constexpr int kMaxHeadDim = 256;
 constexpr int kWavesPerBlock = 4;
 
+// Four consecutive elements in one load; they are used one after the other, in index
+// order, so the sums are those of a loop over single elements.
+typedef __attribute__((ext_vector_type(4))) float f32x4_g;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_g;
+__device__ __forceinline__ f32x4_g load4_g(const float* p) { return *(const f32x4_g*)p; }
+__device__ __forceinline__ f32x4_g load4_g(const bf16_t* p) {
+  const bf16x4_g v = *(const bf16x4_g*)p;
+  return f32x4_g{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
 template <typename T, typename TC>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kernel(AttentionArgs a) {
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
@@ -28,6 +38,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
   const TC* kp = (const TC*)a.k_pages;
   const TC* vp = (const TC*)a.v_pages;
 
+  // head and page sizes in fours (and a cache that starts on 16 bytes): loads of four
+  const bool by4 = hd % 4 == 0 && P % 4 == 0 && (((uintptr_t)kp | (uintptr_t)vp) & 15) == 0;
   for (int d = lane; d < hd; d += kWave) q_s[wave][d] = to_f32(q[d]);
   // a wavefront runs in lockstep and only reads its own rows of LDS: no barrier needed,
   // but the compiler must not reorder the LDS traffic
@@ -46,7 +58,15 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
         row = ((int64_t)page * a.nkv + kvh) * P * hd + j % P;   // of the value column
         const TC* kr = kp + ((int64_t)page * a.nkv + kvh) * P * hd + (int64_t)(j % P) * hd;
         float dot = 0.f;
-        for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
+        if (by4) {
+          for (int d = 0; d < hd; d += 4) {
+            const f32x4_g k4 = load4_g(kr + d);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dot = fmaf(q_s[wave][d + e], k4[e], dot);
+          }
+        } else {
+          for (int d = 0; d < hd; ++d) dot = fmaf(q_s[wave][d], to_f32(kr[d]), dot);
+        }
         s = dot * a.scale;
       }
     }
@@ -61,14 +81,46 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
 #pragma unroll
     for (int r = 0; r < kMaxHeadDim / kWave; ++r) acc[r] *= corr;
     const int n = min(kWave, pos - j0 + 1);
-    for (int jj = 0; jj < n; ++jj) {
-      const int64_t vrow = row_s[wave][jj];
-      if (vrow < 0) continue;
-      const float pj = p_s[wave][jj];
+    if (by4) {
+      // four keys at a time where the group starts at a multiple of four (it then lies in
+      // one page, side by side in each value row), key by key elsewhere (a tile starts at
+      // the first visible key, which a window puts anywhere); in key order either way
+      for (int jj = 0; jj < n; jj += 4) {
+        const int64_t vrow = row_s[wave][jj];
+        const bool whole = jj + 3 < n && vrow >= 0 && ((j0 + jj) & 3) == 0;
+        if (whole) {
 #pragma unroll
-      for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
-        const int d = lane + r * kWave;
-        if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vrow + (int64_t)d * P]), acc[r]);
+          for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+            const int d = lane + r * kWave;
+            if (d < hd) {
+              const f32x4_g v4 = load4_g(vp + vrow + (int64_t)d * P);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[r] = fmaf(p_s[wave][jj + e], v4[e], acc[r]);
+            }
+          }
+        } else {
+          for (int e = 0; e < 4 && jj + e < n; ++e) {
+            const int64_t vr = row_s[wave][jj + e];
+            if (vr < 0) continue;
+            const float pj = p_s[wave][jj + e];
+#pragma unroll
+            for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+              const int d = lane + r * kWave;
+              if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vr + (int64_t)d * P]), acc[r]);
+            }
+          }
+        }
+      }
+    } else {
+      for (int jj = 0; jj < n; ++jj) {
+        const int64_t vrow = row_s[wave][jj];
+        if (vrow < 0) continue;
+        const float pj = p_s[wave][jj];
+#pragma unroll
+        for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+          const int d = lane + r * kWave;
+          if (d < hd) acc[r] = fmaf(pj, to_f32(vp[vrow + (int64_t)d * P]), acc[r]);
+        }
       }
     }
     __builtin_amdgcn_wave_barrier();
