@@ -9,13 +9,13 @@ library, construction raises.
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, Structure, byref, c_float, c_int, c_void_p
+from ctypes import Structure, byref, c_float, c_int, c_void_p
 
 import torch
 
 from tokensprint_amd.kernels.build import build, find_library
 from tokensprint_amd.kernels.dispatch import default_dispatch
-from tokensprint_amd.kernels.stream import NormHint, PreparedRows, UnmergedRows
+from tokensprint_amd.kernels.stream import PreparedRows, UnmergedRows
 
 ABI_VERSION = 1
 _TYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
