@@ -2,6 +2,8 @@
 float32 and bfloat16, at sizes other than the engine's tiny models: widths and
 vocabularies that are no power of two, head sizes in steps of 16, odd head groupings."""
 
+import ctypes
+
 import pytest
 import torch
 
@@ -213,7 +215,7 @@ def test_gemm_tiled(ops, gpu_device, out_dtype, M, N, K):
     ref = x.float() @ w.float().T
     t = dict(rtol=2e-3, atol=2e-3) if out_dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
     first = None
-    for tile in (0, 1, 2, 3, 4):
+    for tile in (0, 1, 2, 3, 4, 5):
         out = ops.gemm_tiled(x, w, out_dtype, tile=tile)
         torch.testing.assert_close(out.float(), ref, **t)
         first = out if first is None else first
@@ -235,7 +237,7 @@ def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
     w[I + I // 3] *= 8                  # and one up column elsewhere
     ref = REF.linear_silu_mul(x, w, torch.bfloat16)
     first = None
-    for tile in (0, 1, 2, 3, 4):
+    for tile in (0, 1, 2, 3, 4, 5):
         out = ops.gemm_tiled(x, w, torch.bfloat16, pair=True, tile=tile)
         torch.testing.assert_close(out.float(), ref.float(), rtol=2e-2, atol=2e-2)
         first = out if first is None else first
@@ -243,6 +245,91 @@ def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
     # the engine's entry takes this kernel from 65 rows on at weights of this size
     if 2 * I * K <= ops.dispatch.tiled_pair_weight:
         assert torch.equal(ops.linear_silu_mul(x, w, torch.bfloat16), first)
+
+
+@pytest.mark.parametrize("M,N,K,next_n,silu", [(2051, 1024, 2048, 3072, True),
+                                               (513, 320, 1024, 400, False),
+                                               (700, 576, 4096, 112, True),
+                                               (1030, 1024, 3072, 4096, False)])
+def test_gemm_tiled_into_stream(ops, gpu_device, M, N, K, next_n, silu):
+    """The tiled product's tail form (adds itself into the float32 stream, hands the stream
+    on times the norm's weight, with the rows' sums of squares in slices) and the scaled
+    form behind it, each against float32 arithmetic on what it was given, every tile the
+    same to the bit; then the two through the provider's entry points against the
+    separate product, add-and-norm and product.  The stream's rows differ a hundredfold
+    in size, so that a factor taken from another row shows."""
+    from tokensprint_amd.kernels.hip_ops import _ptr
+    from tokensprint_amd.kernels.stream import NormHint, PreparedRows
+    bf = torch.bfloat16
+    x = rand((M, K), bf, gpu_device, 60)
+    w = rand((N, K), bf, gpu_device, 61, scale=0.03)
+    resid0 = rand((M, N), torch.float32, gpu_device, 62)
+    resid0 *= torch.logspace(-1, 1, M, device=gpu_device)[torch.randperm(M, device=gpu_device)][:, None]
+    g = rand((N,), torch.float32, gpu_device, 63).abs() + 0.5
+    wn = rand((next_n * (2 if silu else 1), N), bf, gpu_device, 64, scale=0.05)
+    eps = 1e-5
+    delta = (x.float() @ w.float().T)
+    parts = ops.lib.ts_gemm_tiled_tail_parts(N)
+    first = None
+    for tile in (0, 1, 2, 3, 4, 5):
+        resid = resid0.clone()
+        rows = torch.empty(M, N, dtype=bf, device=gpu_device)
+        sumsq = torch.empty(parts, M, dtype=torch.float32, device=gpu_device)
+        ops._call(ops.lib.ts_gemm_tiled_tail_bf16, _ptr(x), _ptr(w), _ptr(resid), _ptr(g), _ptr(rows),
+                  _ptr(sumsq), M, N, K, tile, ops._stream())
+        if first is None:
+            # the product is rounded to bfloat16 before it is added: half an ulp of it off
+            # where the sums' order rounds the other way
+            torch.testing.assert_close(resid - resid0, delta, rtol=1e-2, atol=1e-2)
+            assert torch.equal(rows, (resid * g).to(bf))
+            torch.testing.assert_close(sumsq.double().sum(0), (resid.double() ** 2).sum(1),
+                                       rtol=1e-5, atol=0)
+            first = (resid, rows, sumsq)
+        for got, want in zip((resid, rows, sumsq), first):
+            assert torch.equal(got, want), f"tail tile {tile} differs"
+    resid, rows, sumsq = first
+    rstd = torch.rsqrt((resid.double() ** 2).sum(1, keepdim=True) / N + eps)
+    prod = (rows.double() @ wn.double().T * rstd).float()
+    if silu:
+        gate, up = prod[:, :next_n].to(bf).float(), prod[:, next_n:].to(bf).float()
+        want = gate * torch.sigmoid(gate) * up
+    else:
+        want = prod
+    first_out = None
+    for tile in (0, 1, 2, 3, 4, 5):
+        out = torch.empty(M, next_n, dtype=bf, device=gpu_device)
+        ops._call(ops.lib.ts_gemm_tiled_scaled_bf16, _ptr(rows), _ptr(sumsq), parts, ctypes.c_float(eps),
+                  _ptr(wn), _ptr(out), 1, M, next_n, N, int(silu), tile, ops._stream())
+        torch.testing.assert_close(out.float(), want, rtol=2e-2, atol=2e-2)
+        first_out = out if first_out is None else first_out
+        assert torch.equal(out, first_out), f"scaled tile {tile} differs"
+    # through the provider, where its table sends these sizes to the two forms
+    hint = NormHint(g, eps, wn, silu)
+    if ops._tiled_stream_ok(M, N, K, hint):
+        stream = resid0.clone()
+        prepared = ops.linear_into_stream(x, w, stream, hint)
+        assert isinstance(prepared, PreparedRows)
+        assert torch.equal(stream, resid)
+        out, stream_out = ops.norm_linear(stream, prepared, g, eps, wn, bf, silu_mul=silu)
+        assert torch.equal(out, first_out) and stream_out is stream
+        apart, stream_apart = ops.norm_linear(resid0.clone(), ops.linear(x, w, bf), g, eps, wn, bf,
+                                              silu_mul=silu)
+        torch.testing.assert_close(stream_apart, stream, rtol=1e-2, atol=1e-2)
+        # The two round the normed rows to bfloat16 at different places (before or after the
+        # division by the root mean square), so each is compared with the exact function of
+        # the stream: a product of N terms of size 0.05 with operands 2^-9 off is 0.01 off
+        # and rounded to 2^-9 of itself, and silu(gate) * up carries both factors' errors.
+        s64 = stream.double()
+        h = s64 * torch.rsqrt((s64 ** 2).mean(1, keepdim=True) + eps) * g.double()
+        exact = h @ wn.double().T
+        if silu:
+            gate, up = exact[:, :next_n], exact[:, next_n:]
+            exact, slack = gate * torch.sigmoid(gate) * up, 0.02 * (1 + gate.abs() + up.abs())
+        else:
+            slack = 0.02
+        for name, got in (("fused", out), ("apart", apart)):
+            excess = (got.double() - exact).abs() - slack - 0.01 * exact.abs()
+            assert excess.max().item() <= 0, f"{name}: {excess.max().item()} beyond the bound"
 
 
 def test_gemm_tiled_refuses_what_it_cannot_take(ops, gpu_device):

@@ -5,6 +5,7 @@
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 
 constexpr int kIterK = 128;   // K elements a wave consumes per iteration (4 MFMA steps)
 

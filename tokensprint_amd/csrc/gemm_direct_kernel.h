@@ -5,7 +5,6 @@
 #include <type_traits>
 #include "gemm_common.h"
 
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 
 // The lane's 16-byte register moved n lanes down its row of 16 lanes (lane i takes lane
 // i + n's; the top n lanes get zeros).

@@ -42,6 +42,12 @@ class Dispatch:
     # is neither written nor read; at the 8B shape 0.85 to 1.07, at the 32B shape 1.02 to
     # 1.20, the library's product itself being 10 to 20 % ahead at large sizes.
     tiled_pair_weight: int = 1 << 23
+    #: rows from which, and elements of a weight [N, K] up to which, the product that ends a
+    #: sub-layer is the LDS-tiled kernel's tail form (it adds itself into the float32 stream
+    #: and prepares the rows for the norm behind it, whose product then takes the scaled
+    #: form) instead of the library's product and a norm kernel.
+    tiled_stream_rows: int = 512
+    tiled_stream_weight: int = 1 << 23
 
     # ---- attention.  Measured at 16 query / 8 key-value heads of 128, page size 16.
     #: workgroups (entries x key/value heads) up to which a decode step takes the decode

@@ -396,6 +396,17 @@ class HipOps:
         if weight.shape[1] != K:
             raise ValueError(f"linear_into_stream: x has {K} columns, weight has {weight.shape[1]}")
         next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
+        if self._tiled_stream_ok(M, N, K, hint):
+            # a prompt's portion: the LDS-tiled product in its tail form
+            self._check("resid", resid, torch.float32, shape=(M, N))
+            self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
+            rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
+            sumsq = torch.empty(self.lib.ts_gemm_tiled_tail_parts(N), M, dtype=torch.float32,
+                                device=self.device)
+            self._call(self.lib.ts_gemm_tiled_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
+                       _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, 0,
+                       self._stream())
+            return PreparedRows(rows, sumsq, hint)
         parts = self.lib.ts_gemm_tail_parts(M, N)
         if hint.weight.shape[1] != N or self._library_rows(M, N, K) \
                 or self._library_rows(M, next_n, N) \
@@ -409,6 +420,18 @@ class HipOps:
         self._call(self.lib.ts_gemm_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
                    _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, self._stream())
         return PreparedRows(rows, sumsq, hint)
+
+    def _tiled_stream_ok(self, M, N, K, hint):
+        """Whether the product [M, K] x [N, K] that ends a sub-layer, and the hinted norm
+        and product behind it, are the LDS-tiled kernel's tail and scaled forms."""
+        d = self.dispatch
+        if M < d.tiled_stream_rows or hint.weight.shape[1] != N \
+                or N * K > d.tiled_stream_weight or hint.weight.numel() > d.tiled_pair_weight:
+            return False
+        next_n = hint.weight.shape[0] // 2 if hint.silu_mul else hint.weight.shape[0]
+        return (self.lib.ts_gemm_tiled_tail_fits(M, N, K) == 1
+                and self.lib.ts_gemm_tiled_scaled_fits(
+                    M, next_n, N, int(hint.silu_mul), self.lib.ts_gemm_tiled_tail_parts(N)) == 1)
 
     def _merged_into_stream(self, unmerged, x, weight, resid, hint):
         """`linear_into_stream` over an attention output that is still unmerged: one kernel
@@ -450,6 +473,11 @@ class HipOps:
         if out_dtype not in (torch.bfloat16, torch.float32) or (silu_mul and out_dtype != torch.bfloat16):
             raise ValueError(f"norm_linear: prepared rows cannot give {out_dtype}")
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
+        if M >= self.dispatch.tiled_stream_rows:      # prepared by the tiled tail form
+            self._call(self.lib.ts_gemm_tiled_scaled_bf16, _ptr(prepared.rows),
+                       _ptr(prepared.sumsq), prepared.sumsq.shape[0], c_float(eps), _ptr(weight),
+                       _ptr(out), _TYPE_CODE[out_dtype], M, N, K, int(silu_mul), 0, self._stream())
+            return out, resid
         self._call(self.lib.ts_gemm_scaled_bf16, _ptr(prepared.rows), _ptr(prepared.sumsq),
                    prepared.sumsq.shape[0], c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
                    int(silu_mul), self._stream())
