@@ -37,7 +37,7 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   // whatever its lanes ask for, and that rate, not the bytes, bounds these products.  An
   // operand with fewer than 16 rows (AR rows of A that exist, CW rows of W that this
   // workgroup owns) is therefore loaded with its 16 row lanes split into 16/AR (16/CW)
-  // sets that fetch consecutive 8-element pieces of K, one instruction instead of
+  // sets that fetch the pieces of 16/AR consecutive products, one instruction instead of
   // several, and the piece a product needs is moved down to the first rows' lanes (a DPP
   // move; the other rows of the operand only produce results that nobody stores).
   static_assert((CW == 16 || CW == 8 || CW == 4) && (AR == 16 || AR == 8 || AR == 4), "rows");
@@ -49,7 +49,12 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   // slices of the sums of squares a lane adds per tile (16 registers in all)
   constexpr int kPartLoads = SCALED ? 16 / MT : 1;
   constexpr int kStep = S * 32;          // K elements of one step
-  constexpr int kLane = S * 8;           // of which a lane holds this many, contiguous
+  // Where a lane's 8-element pieces of a step lie: piece s of lane group g at
+  // s * kPiece + g * kGroup elements, so that the four lanes of a row read 64 contiguous
+  // bytes with one instruction (a lane with its S pieces side by side had an instruction
+  // touch twice as many cache lines: 0.1 to 0.7 us more per product, measured at 8 to 64
+  // rows).  A and W take the same places, so the products' pairs are the same.
+  constexpr int kGroup = 8, kPiece = 32;
   constexpr int NW = PAIR ? 2 : 1;
   __shared__ f32x4 red[(WK - 1) * NW * MT * kWave];
   __shared__ float ss_part[(NORM || SCALED) ? WK * MT * 16 : 1];
@@ -60,12 +65,12 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   const int n0 = blockIdx.x * CW;
   const int m_base = blockIdx.y * (MT * 16);
   // rows past the end read the last row again; their results are never stored
-  const int64_t w_off = (int64_t)min(n0 + r % CW, N - 1) * K + g * kLane + (r / CW) * 8;
+  const int64_t w_off = (int64_t)min(n0 + r % CW, N - 1) * K + g * kGroup + (r / CW) * kPiece;
   const bf16_t* wrow = a.W + w_off;
   int64_t a_off[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
-    a_off[mt] = (int64_t)min(m_base + mt * 16 + r % AR, M - 1) * K + g * kLane + (r / AR) * 8;
+    a_off[mt] = (int64_t)min(m_base + mt * 16 + r % AR, M - 1) * K + g * kGroup + (r / AR) * kPiece;
   // without a delta the loads read the stream's own memory and the values are dropped:
   // no branch around a load
   const bool has_delta = NORM && a.delta != nullptr;
@@ -141,31 +146,31 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char merged_rows[];
   const int row_pieces = K / 8 + 1;
   const bf16x8* a_row = (const bf16x8*)merged_rows + min(m_base + r % AR, M - 1) * row_pieces +
-                        (g * kLane + (r / AR) * 8) / 8;
+                        (g * kGroup + (r / AR) * kPiece) / 8;
   auto load = [&](Step& st, int kb, bool of_w = true, bool of_a = true) {
 #pragma unroll
     for (int s = 0; s < S; ++s) {
       if (s % GW == 0 && of_w) {
 #pragma unroll
         for (int w = 0; w < NW; ++w)
-          st.w[w][s / GW] = *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8);
+          st.w[w][s / GW] = *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * kPiece);
       }
       if (!of_a) continue;
       if constexpr (MERGE) {
-        if (s % GA == 0) st.x[0][s / GA] = a_row[(kb + s * 8) / 8];
+        if (s % GA == 0) st.x[0][s / GA] = a_row[(kb + s * kPiece) / 8];
       } else if constexpr (NORM) {
-        const float* rp = a.resid_in + a_off[0] + kb + s * 8;
+        const float* rp = a.resid_in + a_off[0] + kb + s * kPiece;
         st.rs[s][0] = *(const f32x4*)rp;
         st.rs[s][1] = *(const f32x4*)(rp + 4);
-        st.d[s] = *(const bf16x8*)(dbase + a_off[0] + kb + s * 8);
-        const float* np = a.norm_w + g * kLane + kb + s * 8;
+        st.d[s] = *(const bf16x8*)(dbase + a_off[0] + kb + s * kPiece);
+        const float* np = a.norm_w + g * kGroup + kb + s * kPiece;
         st.nw[s][0] = *(const f32x4*)np;
         st.nw[s][1] = *(const f32x4*)(np + 4);
       } else {
         if (s % GA == 0) {
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            st.x[mt][s / GA] = *(const bf16x8*)(a.A + a_off[mt] + kb + s * 8);
+            st.x[mt][s / GA] = *(const bf16x8*)(a.A + a_off[mt] + kb + s * kPiece);
         }
       }
     }
@@ -174,30 +179,30 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   auto load_tail = [&](Step& st, int kb) {
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-      const bool ok = kb + g * kLane + s * 8 < K;
+      const bool ok = kb + g * kGroup + s * kPiece < K;
       if (s % GW == 0) {
-        const bool ok_w = kb + g * kLane + (s + r / CW) * 8 < K;
+        const bool ok_w = kb + g * kGroup + (s + r / CW) * kPiece < K;
 #pragma unroll
         for (int w = 0; w < NW; ++w)
-          st.w[w][s / GW] = ok_w ? *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * 8) : zero;
+          st.w[w][s / GW] = ok_w ? *(const bf16x8*)(wrow + (int64_t)w * N * K + kb + s * kPiece) : zero;
       }
       if constexpr (MERGE) {
         if (s % GA == 0)
-          st.x[0][s / GA] = kb + g * kLane + (s + r / AR) * 8 < K ? a_row[(kb + s * 8) / 8] : zero;
+          st.x[0][s / GA] = kb + g * kGroup + (s + r / AR) * kPiece < K ? a_row[(kb + s * kPiece) / 8] : zero;
       } else if constexpr (NORM) {
-        const float* rp = a.resid_in + a_off[0] + kb + s * 8;
+        const float* rp = a.resid_in + a_off[0] + kb + s * kPiece;
         st.rs[s][0] = ok ? *(const f32x4*)rp : fzero;
         st.rs[s][1] = ok ? *(const f32x4*)(rp + 4) : fzero;
-        st.d[s] = ok ? *(const bf16x8*)(dbase + a_off[0] + kb + s * 8) : zero;
-        const float* np = a.norm_w + g * kLane + kb + s * 8;
+        st.d[s] = ok ? *(const bf16x8*)(dbase + a_off[0] + kb + s * kPiece) : zero;
+        const float* np = a.norm_w + g * kGroup + kb + s * kPiece;
         st.nw[s][0] = ok ? *(const f32x4*)np : fzero;
         st.nw[s][1] = ok ? *(const f32x4*)(np + 4) : fzero;
       } else {
         if (s % GA == 0) {
-          const bool ok_a = kb + g * kLane + (s + r / AR) * 8 < K;
+          const bool ok_a = kb + g * kGroup + (s + r / AR) * kPiece < K;
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
-            st.x[mt][s / GA] = ok_a ? *(const bf16x8*)(a.A + a_off[mt] + kb + s * 8) : zero;
+            st.x[mt][s / GA] = ok_a ? *(const bf16x8*)(a.A + a_off[mt] + kb + s * kPiece) : zero;
         }
       }
     }

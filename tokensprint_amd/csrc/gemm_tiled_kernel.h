@@ -78,6 +78,18 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// Waits until at most the loads of `younger` K steps (of LOADS each; at most MOST steps)
+// are in flight.
+template <int LOADS, int MOST>
+__device__ __forceinline__ void wait_steps(int younger) {
+  if constexpr (MOST <= 0) {
+    wait_loads<0>();
+  } else {
+    if (younger >= MOST) wait_loads<LOADS * MOST>();
+    else wait_steps<LOADS, MOST - 1>(younger);
+  }
+}
+
 template <int BM, int BN, int GM, int GN, int STAGES, bool PAIR, typename TO, int FORM = kPlain>
 __global__ __launch_bounds__(64 * GM * GN, 1) void gemm_tiled_kernel(TiledArgs g) {
   static_assert(!(FORM == kTail && PAIR), "the product that ends a sub-layer has one weight");
@@ -90,7 +102,7 @@ __global__ __launch_bounds__(64 * GM * GN, 1) void gemm_tiled_kernel(TiledArgs g
   constexpr int LA = BM / (8 * NW), LW = BN / (8 * NW);   // load instructions a wave issues per step
   constexpr int LOADS = LA + LW;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
-  static_assert(STAGES >= 2 && STAGES <= 4, "the waits below are written for 2 to 4 buffers");
+  static_assert(STAGES >= 2 && STAGES <= 8, "a ring of 2 to 8 buffers");
   static_assert(LOADS * (STAGES - 1) < 64, "the load counter has six bits");
   extern __shared__ __attribute__((aligned(1024))) unsigned char tiled_lds[];
 
@@ -255,10 +267,7 @@ __global__ __launch_bounds__(64 * GM * GN, 1) void gemm_tiled_kernel(TiledArgs g
       for (int s = 0; s < STAGES; ++s) {
         const int kt = kt0 + s;
         if (kt >= KT) break;
-        const int younger = min(STAGES - 2, KT - 1 - kt);
-        if (younger >= 2) wait_loads<LOADS * (STAGES >= 4 ? 2 : 0)>();
-        else if (younger == 1) wait_loads<LOADS * (STAGES >= 3 ? 1 : 0)>();
-        else wait_loads<0>();
+        wait_steps<LOADS, STAGES - 2>(min(STAGES - 2, KT - 1 - kt));
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -312,10 +321,7 @@ __global__ __launch_bounds__(64 * GM * GN, 1) void gemm_tiled_kernel(TiledArgs g
         const bool more = kt + 1 < KT;
         if (more) {
           // step kt + 1 has arrived when at most the younger steps' loads are in flight
-          const int younger = min(STAGES - 2, KT - 2 - kt);
-          if (younger >= 2) wait_loads<LOADS * (STAGES >= 4 ? 2 : 0)>();
-          else if (younger == 1) wait_loads<LOADS * (STAGES >= 3 ? 1 : 0)>();
-          else wait_loads<0>();
+          wait_steps<LOADS, STAGES - 2>(min(STAGES - 2, KT - 2 - kt));
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // this wave has read step kt
           __builtin_amdgcn_s_barrier();
           asm volatile("" ::: "memory");
