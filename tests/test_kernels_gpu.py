@@ -415,7 +415,8 @@ def test_linear_into_stream_then_norm_linear(ops, gpu_device, silu, M, W, K, N):
         x.double().pow(2).mean().sqrt() * wo.double().pow(2).mean().sqrt())
     assert ((r.double() - (resid.double() + delta)).abs() <= 1.01 * dnoise + 1e-6).all()
     xs = r.double()
-    assert torch.allclose(prepared.sumsq.double().sum(0), xs.pow(2).sum(-1), rtol=1e-5)
+    assert prepared.sumsq.shape == (M, -(-prepared.slices // 4) * 4)     # a row's slices side by side
+    assert torch.allclose(prepared.sumsq[:, :prepared.slices].double().sum(1), xs.pow(2).sum(-1), rtol=1e-5)
     torch.testing.assert_close(prepared.rows.float(), (r * nw).to(bf).float(), rtol=2 ** -7, atol=1e-30)
     h = xs * torch.rsqrt(xs.pow(2).mean(-1, keepdim=True) + 1e-5) * nw.double()
     y = h @ w.double().T
@@ -879,7 +880,8 @@ def test_output_projection_merges_the_key_splits_itself(ops, gpu_device, monkeyp
     assert prep_ref is not None and prep_new is not None
     assert torch.equal(resid_new, resid_ref)
     assert torch.equal(prep_new.rows, prep_ref.rows)
-    assert torch.equal(prep_new.sumsq, prep_ref.sumsq)
+    assert prep_new.slices == prep_ref.slices
+    assert torch.equal(prep_new.sumsq[:, :prep_new.slices], prep_ref.sumsq[:, :prep_ref.slices])
     # deferred, then met by another call: merged first, the same attention output
     mine = type(cache)(cache.group, cache.page_size, cache.num_pages,
                        cache.k_pages.clone(), cache.v_pages.clone())

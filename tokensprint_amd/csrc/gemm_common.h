@@ -51,10 +51,10 @@ struct DirectArgs {
   float* resid;             // [M, N]
   const float* tail_w;      // [N]
   bf16_t* prepared;         // [M, N] out
-  float* sumsq_out;         // [gemm_direct_tail_parts(M, N)][M] out
+  float* sumsq_out;         // [M][gemm_direct_tail_parts(M, N) rounded up to 4] out
   // scaled form (sumsq set): A holds such prepared rows; C's rows are divided by the
   // root mean square that the slices of sums of squares give
-  const float* sumsq;       // [parts][M]
+  const float* sumsq;       // [M][parts rounded up to 4]
   int parts;
   // merged form (merge_o set; tail form, at most 16 rows): A is not stored either but is a
   // decode step's attention output still lying in the partial sums of its key splits, as

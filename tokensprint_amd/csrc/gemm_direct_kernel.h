@@ -46,8 +46,8 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   constexpr int GW = 16 / CW, GA = 16 / AR;          // pieces per load instruction
   static_assert(S % GW == 0 && S % GA == 0, "a step holds whole instructions");
   static_assert(!(NORM && SCALED) && !(TAIL && (NORM || SCALED || PAIR)), "one form at a time");
-  // slices of the sums of squares a lane adds per tile (16 registers in all)
-  constexpr int kPartLoads = SCALED ? 16 / MT : 1;
+  // slices of the sums of squares a lane adds per tile (16 registers in all), four to a load
+  constexpr int kPartLoads = SCALED ? 4 / MT : 1;
   constexpr int kStep = S * 32;          // K elements of one step
   // Where a lane's 8-element pieces of a step lie: piece s of lane group g at
   // s * kPiece + g * kGroup elements, so that the four lanes of a row read 64 contiguous
@@ -108,9 +108,11 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
       tail_x[mt] = *(const f32x4*)(a.resid + (int64_t)min(m_base + mt * 16 + r, M - 1) * N + tail_n);
     tail_w4 = *(const f32x4*)(a.tail_w + tail_n);
   }
-  // scaled form: slice j of a row's sum of squares goes to wave (j / 4) % WK, lane group
-  // j % 4; a slice past the last reads the last again and is dropped
-  float part[MT][kPartLoads];
+  // scaled form: a row's slices lie side by side (rows of `parts` rounded up to four);
+  // four of them, 4 j .. 4 j + 3, go to wave (j / 4) % WK, lane group j % 4 in one load; a
+  // four past the last reads the last again and is dropped
+  const int part_stride = (a.parts + 3) & ~3;
+  f32x4 part[MT][kPartLoads];
   auto load_parts = [&]() {
     if constexpr (SCALED) {
 #pragma unroll
@@ -118,7 +120,8 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
 #pragma unroll
         for (int i = 0; i < kPartLoads; ++i) {
           const int j = (i * WK + wk) * 4 + g;
-          part[mt][i] = a.sumsq[(int64_t)min(j, a.parts - 1) * M + min(m_base + mt * 16 + r, M - 1)];
+          part[mt][i] = *(const f32x4*)(a.sumsq + (int64_t)min(m_base + mt * 16 + r, M - 1) * part_stride +
+                                        4 * min(j, part_stride / 4 - 1));
         }
     }
   };
@@ -421,7 +424,10 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
     for (int mt = 0; mt < MT; ++mt) {
       float sq = 0.f;
 #pragma unroll
-      for (int i = 0; i < kPartLoads; ++i) sq += ((i * WK + wk) * 4 + g < a.parts) ? part[mt][i] : 0.f;
+      for (int i = 0; i < kPartLoads; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          sq += (((i * WK + wk) * 4 + g) * 4 + e < a.parts) ? part[mt][i][e] : 0.f;
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);
       if (g == 0) ss_part[(wk * MT + mt) * 16 + r] = sq;
@@ -482,7 +488,7 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
       sq = ok ? sq : 0.f;
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);
-      if (g == 0 && m < M) a.sumsq_out[(int64_t)blockIdx.x * M + m] = sq;
+      if (g == 0 && m < M) a.sumsq_out[(int64_t)m * (((int)gridDim.x + 3) & ~3) + blockIdx.x] = sq;
     }
     return;
   }

@@ -464,8 +464,9 @@ extern "C" int ts_norm_gemm_mfma_bf16(const float* resid_in, const void* delta, 
 //
 // ts_gemm_tail_bf16: resid[M, N] += bf16(A[M, K] W[N, K]^T) in place (float32), and for
 // the RMSNorm with weight norm_w that follows: prepared[M, N] = bf16(resid * norm_w) and
-// sumsq[ts_gemm_tail_parts(M, N)][M], each row's sum of squares of resid over a slice of
-// its columns (16, or fewer where the product is spread over more workgroups).
+// sumsq[M][ts_gemm_tail_parts(M, N) rounded up to 4], each row's sum of squares of resid
+// over a slice of its columns (16, or fewer where the product is spread over more
+// workgroups); what lies beyond a row's slices is not written.
 extern "C" int ts_gemm_tail_fits(int M, int N, int K) { return gemm_direct_tail_fits(M, N, K); }
 extern "C" int ts_gemm_tail_parts(int M, int N) { return gemm_direct_tail_parts(M, N); }
 
@@ -487,8 +488,8 @@ extern "C" int ts_gemm_tail_bf16(const void* a, const void* w, float* resid, con
   return 0;
 }
 
-// ts_gemm_scaled_bf16: C[M, N] = (prepared[M, K] W[N, K]^T) * rsqrt(sum_j sumsq[j][m] / K + eps)
-// for sumsq[parts][M]; pair as in ts_gemm_mfma_bf16.
+// ts_gemm_scaled_bf16: C[M, N] = (prepared[M, K] W[N, K]^T) * rsqrt(sum_j sumsq[m][j] / K + eps)
+// for sumsq[M][parts rounded up to 4] (16-byte aligned); pair as in ts_gemm_mfma_bf16.
 extern "C" int ts_gemm_scaled_fits(int M, int N, int K, int pair, int parts) {
   return gemm_direct_scaled_fits(M, N, K, pair != 0, parts);
 }
@@ -499,7 +500,8 @@ extern "C" int ts_gemm_scaled_bf16(const void* prepared, const float* sumsq, int
   if (M <= 0 || N <= 0) return 0;
   if (!gemm_direct_scaled_fits(M, N, K, pair != 0, parts))
     TS_FAIL("gemm_scaled: M=%d, N=%d, K=%d is not a product the scaled form takes", M, N, K);
-  if (((uintptr_t)prepared | (uintptr_t)w) & 15) TS_FAIL("gemm_scaled: operands must be 16-byte aligned");
+  if (((uintptr_t)prepared | (uintptr_t)w | (uintptr_t)sumsq) & 15)
+    TS_FAIL("gemm_scaled: operands must be 16-byte aligned");
   if (!prepared || !sumsq || !w || !c) TS_FAIL("gemm_scaled: null operand");
   DirectArgs da = {};
   da.A = (const bf16_t*)prepared; da.W = (const bf16_t*)w; da.C = c; da.M = M; da.N = N; da.K = K;

@@ -406,7 +406,7 @@ class HipOps:
             self._call(self.lib.ts_gemm_tiled_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
                        _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, 0,
                        self._stream())
-            return PreparedRows(rows, sumsq, hint)
+            return PreparedRows(rows, sumsq, sumsq.shape[0], hint)
         parts = self.lib.ts_gemm_tail_parts(M, N)
         if hint.weight.shape[1] != N or self._library_rows(M, N, K) \
                 or self._library_rows(M, next_n, N) \
@@ -416,10 +416,10 @@ class HipOps:
         self._check("resid", resid, torch.float32, shape=(M, N))
         self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
         rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
-        sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
+        sumsq = torch.empty(M, -(-parts // 4) * 4, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_gemm_tail_bf16, _ptr(x), _ptr(weight), _ptr(resid),
                    _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N, K, self._stream())
-        return PreparedRows(rows, sumsq, hint)
+        return PreparedRows(rows, sumsq, parts, hint)
 
     def _tiled_stream_ok(self, M, N, K, hint):
         """Whether the product [M, K] x [N, K] that ends a sub-layer, and the hinted norm
@@ -452,14 +452,14 @@ class HipOps:
         self._check("resid", resid, torch.float32, shape=(M, N))
         self._check("norm weight", hint.norm_weight, torch.float32, shape=(N,))
         rows = torch.empty(M, N, dtype=torch.bfloat16, device=self.device)
-        sumsq = torch.empty(parts, M, dtype=torch.float32, device=self.device)
+        sumsq = torch.empty(M, -(-parts // 4) * 4, dtype=torch.float32, device=self.device)
         self._call(self.lib.ts_gemm_tail_merged_bf16, _ptr(unmerged.partial_o),
                    _ptr(unmerged.partial_ml), _ptr(unmerged.positions),
                    unmerged.args.num_splits, a.nq, a.nkv, a.hd,
                    0 if unmerged.window is None else int(unmerged.window), _ptr(weight),
                    _ptr(resid), _ptr(hint.norm_weight), _ptr(rows), _ptr(sumsq), M, N,
                    self._stream())
-        return PreparedRows(rows, sumsq, hint)
+        return PreparedRows(rows, sumsq, parts, hint)
 
     def _prepared_linear(self, resid, prepared, norm_weight, eps, weight, out_dtype, silu_mul):
         hint = prepared.hint
@@ -475,11 +475,11 @@ class HipOps:
         out = torch.empty(M, N, dtype=out_dtype, device=self.device)
         if M >= self.dispatch.tiled_stream_rows:      # prepared by the tiled tail form
             self._call(self.lib.ts_gemm_tiled_scaled_bf16, _ptr(prepared.rows),
-                       _ptr(prepared.sumsq), prepared.sumsq.shape[0], c_float(eps), _ptr(weight),
+                       _ptr(prepared.sumsq), prepared.slices, c_float(eps), _ptr(weight),
                        _ptr(out), _TYPE_CODE[out_dtype], M, N, K, int(silu_mul), 0, self._stream())
             return out, resid
         self._call(self.lib.ts_gemm_scaled_bf16, _ptr(prepared.rows), _ptr(prepared.sumsq),
-                   prepared.sumsq.shape[0], c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
+                   prepared.slices, c_float(eps), _ptr(weight), _ptr(out), _TYPE_CODE[out_dtype], M, N, K,
                    int(silu_mul), self._stream())
         return out, resid
 

@@ -27,12 +27,15 @@ class NormHint:
 class PreparedRows:
     """A sub-layer's output already added into the residual stream, and the stream handed
     on prepared for the RMSNorm of `hint`: `rows` [M, K] = stream * norm weight (bfloat16,
-    not yet divided by the row's root mean square) and `sumsq` [slices, M], the
-    rows' sums of squares in slices of columns (as wide as the producing kernel makes them).  Stands where the stream's `delta` does,
-    and only the provider's `norm_linear` with the hinted norm and weight takes it."""
+    not yet divided by the row's root mean square) and `sumsq`, the rows' sums of squares
+    in `slices` slices of columns, laid out as the producing kernel and its counterpart
+    agree ([M, slices rounded up to four] from the kernels for few rows, [slices, M] from
+    the tiled product's).  Stands where the stream's `delta` does, and only the provider's
+    `norm_linear` with the hinted norm and weight takes it."""
 
     rows: torch.Tensor
     sumsq: torch.Tensor
+    slices: int
     hint: NormHint
 
 
