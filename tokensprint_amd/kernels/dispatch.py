@@ -45,7 +45,10 @@ class Dispatch:
     #: rows from which, and elements of a weight [N, K] up to which, the product that ends a
     #: sub-layer is the LDS-tiled kernel's tail form (it adds itself into the float32 stream
     #: and prepares the rows for the norm behind it, whose product then takes the scaled
-    #: form) instead of the library's product and a norm kernel.
+    #: form) instead of the library's product and a norm kernel.  Plain products of such
+    #: sizes (a model's first layer, whose norm nothing prepares) take the tiled kernel too:
+    #: the same time on the GPU (22.5 against 22.4 us for qkv at 2,048 rows) and a fifth of
+    #: the library call's 20 to 30 us on the host, which the GPU waits for at a step's start.
     tiled_stream_rows: int = 512
     tiled_stream_weight: int = 1 << 23
 

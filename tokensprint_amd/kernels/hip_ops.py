@@ -260,6 +260,10 @@ class HipOps:
         N = weight.shape[0]
         if weight.shape[1] != K:
             raise ValueError(f"linear: x has {K} columns, weight has {weight.shape[1]}")
+        if self._tiled_plain_ok(M, N, K, x.dtype, weight.dtype, out_dtype):
+            # a prompt's portion at small weights: as fast as the library's product on the
+            # GPU and a fifth of its cost on the host (which a step's first layer waits for)
+            return self.gemm_tiled(x, weight, out_dtype)
         if self._library_ok(x, weight):
             # the library's float32 sums leave in the type asked for: bfloat16 activations,
             # float32 logits at the output head (not rounded to bfloat16 and widened, so
@@ -320,6 +324,13 @@ class HipOps:
                 and out_dtype == torch.bfloat16 and weight.numel() <= self.dispatch.tiled_pair_weight
                 and self._library_rows(M, weight.shape[0], K)
                 and self.lib.ts_gemm_tiled_fits(M, inner, K, 1) == 1)
+
+    def _tiled_plain_ok(self, M, N, K, x_dtype, w_dtype, out_dtype):
+        d = self.dispatch
+        return (x_dtype == torch.bfloat16 and w_dtype == torch.bfloat16
+                and out_dtype in (torch.bfloat16, torch.float32)
+                and M >= d.tiled_stream_rows and N * K <= d.tiled_stream_weight
+                and self.lib.ts_gemm_tiled_fits(M, N, K, 0) == 1)
 
     def _library_ok(self, x, weight, out_dtype=None):
         if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
@@ -833,8 +844,7 @@ class HipOps:
             # kernel's balance only, never for what it computes (it reads positions and
             # lengths on the device).
             tiles = [(entry, entry, 1) for entry in range(batch.num_entries)]
-            host = torch.tensor(tiles, dtype=torch.int32)
-            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
+            batch.plans[key] = (self._upload_ints(tiles), len(tiles))
         if key not in batch.plans:
             tiles, keys = [], []
             first = 0
@@ -847,9 +857,32 @@ class HipOps:
             if longest_first:
                 order = sorted(range(len(tiles)), key=lambda i: -keys[i])
                 tiles = [tiles[i] for i in order]
-            host = torch.tensor(tiles, dtype=torch.int32)
-            batch.plans[key] = (host.to(self.device, non_blocking=True), len(tiles))
+            batch.plans[key] = (self._upload_ints(tiles), len(tiles))
         return batch.plans[key]
+
+    def _upload_ints(self, rows):
+        """A list of equally long int tuples as an int32 device tensor, copied out of pinned
+        memory (a copy out of pageable memory holds the host until it is done, and the step's
+        first attention call, which the GPU is waiting for, makes this list).  Four buffers
+        in turn, each free again once its last copy has been made."""
+        host = torch.tensor(rows, dtype=torch.int32)
+        if self.device.type != "cuda":
+            return host.to(self.device)
+        turn = self._staging_turn = (getattr(self, "_staging_turn", -1) + 1) % 4
+        if not hasattr(self, "_staging"):
+            self._staging = [None] * 4
+        slot = self._staging[turn]
+        if slot is None or slot[0].numel() < host.numel():
+            slot = (torch.empty(max(host.numel(), 1 << 14), dtype=torch.int32, pin_memory=True),
+                    torch.cuda.Event())
+            self._staging[turn] = slot
+        else:
+            slot[1].synchronize()
+        pinned = slot[0][:host.numel()].view(host.shape)
+        pinned.copy_(host)
+        dev = pinned.to(self.device, non_blocking=True)
+        slot[1].record()
+        return dev
 
     def _fill_attention_args(self, a, q, out, batch, table, cache, num_heads, num_kv_heads,
                              head_dim, scale, window):
