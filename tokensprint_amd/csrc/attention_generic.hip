@@ -2,9 +2,12 @@
 // float32 or bfloat16 storage, float32 arithmetic throughout: the attention of the
 // float32 path and of shapes the matrix-core kernels do not take.
 //
-// One wavefront per (query token, query head).  Keys are walked in tiles of 64 starting
-// at the first visible key, so the partition, and with it the rounding, depends only on
-// the token's position and the window, never on how the step was cut or batched.
+// One workgroup of four wavefronts per (query token, query head).  Keys are cut into tiles
+// of 64 starting at the first visible key; wavefront w walks tiles w, w + 4, ... and the
+// four partial results are merged in wavefront order, so the partition, and with it the
+// rounding, depends only on the token's position and the window, never on how the step was
+// cut or batched.  (A decode step of few requests has few such pairs: with a wavefront
+// each, 32 of 256 compute units worked.)
 #include "attention.h"
 
 constexpr int kMaxHeadDim = 256;
@@ -25,9 +28,10 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
   __shared__ float p_s[kWavesPerBlock][kWave];
   __shared__ int64_t row_s[kWavesPerBlock][kWave];
+  __shared__ float m_s[kWavesPerBlock], l_s[kWavesPerBlock];
+  __shared__ float acc_s[kWavesPerBlock][kMaxHeadDim];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int64_t item = (int64_t)blockIdx.x * kWavesPerBlock + wave;
-  if (item >= (int64_t)a.num_tokens * a.nq) return;   // whole wave leaves together
+  const int64_t item = blockIdx.x;
   const int t = (int)(item / a.nq), h = (int)(item % a.nq);
   const int kvh = h / (a.nq / a.nkv);
   const int hd = a.hd, P = a.page_size;
@@ -47,7 +51,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
 
   float m = -INFINITY, l = 0.f;
   float acc[kMaxHeadDim / kWave] = {};
-  for (int j0 = lo; j0 <= pos; j0 += kWave) {
+  for (int j0 = lo + wave * kWave; j0 <= pos; j0 += kWavesPerBlock * kWave) {
     const int j = j0 + lane;
     const bool valid = j <= pos;
     float s = -INFINITY;
@@ -126,12 +130,35 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void attention_generic_kerne
     __builtin_amdgcn_wave_barrier();
     m = m_new;
   }
+  // the wavefronts' partial results, merged by the first in wavefront order
+  if (lane == 0) { m_s[wave] = m; l_s[wave] = l; }
+#pragma unroll
+  for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
+    const int d = lane + r * kWave;
+    if (d < hd) acc_s[wave][d] = acc[r];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) m_all = fmaxf(m_all, m_s[w]);
+  float weight[kWavesPerBlock];
+  l = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    weight[w] = m_s[w] == -INFINITY ? 0.f : expf(m_s[w] - m_all);     // a wavefront without keys
+    l += l_s[w] * weight[w];
+  }
   T* o = (T*)a.out + item * hd;
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
   for (int r = 0; r < kMaxHeadDim / kWave; ++r) {
     const int d = lane + r * kWave;
-    if (d < hd) o[d] = from_f32<T>(acc[r] * inv);
+    if (d >= hd) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) sum += weight[w] == 0.f ? 0.f : acc_s[w][d] * weight[w];
+    o[d] = from_f32<T>(sum * inv);
   }
 }
 
@@ -151,8 +178,7 @@ extern "C" int ts_attention_generic(const AttentionArgs* args, int act_type, int
   AttentionArgs a = *args;
   if (a.num_tokens <= 0) return 0;
   if (ts_check_attention_args(a, "attention_generic")) return -1;
-  const int64_t items = (int64_t)a.num_tokens * a.nq;
-  const int64_t blocks = (items + kWavesPerBlock - 1) / kWavesPerBlock;
+  const int64_t blocks = (int64_t)a.num_tokens * a.nq;       // a workgroup per token and head
   if (blocks > 2147483647LL) TS_FAIL("attention_generic: too many tokens");
   TS_DISPATCH_TYPE(act_type, T, TS_DISPATCH_TYPE(cache_type, TC,
       hipLaunchKernelGGL((attention_generic_kernel<T, TC>), dim3((unsigned)blocks),
