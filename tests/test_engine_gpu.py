@@ -245,3 +245,24 @@ def test_decode_lanes_on_both_sides_of_each_kernel_choice(wide_bfloat16, lanes, 
                 f"{lanes} lanes, step {step}, position {pos}: {(row - ref[pos]).abs().max():.3e}"
         for item in live:
             item[1] += 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_long_prompt_through_the_kernels_of_many_rows(dtype, tmp_path, gpu_device):
+    """A prompt of 777 tokens through a small model whose sizes (hidden 320, inner 768:
+    multiples of 64 that are no powers of two) the LDS-tiled products take: whole (in
+    bfloat16 the products carry the stream's add and the norm from 512 rows on, and the
+    wide attention kernel takes the step) and in portions of 477 and 300 (the separate
+    kernels), both against the plain implementation."""
+    from helpers import qwen3_config
+    cfg = qwen3_config(hidden=320, layers=3, heads=4, kv_heads=2, head_dim=64, inter=768,
+                       vocab=1000, eps=1e-6, theta=1e4, tied=True, max_pos=1024)
+    write_random_model(tmp_path, cfg, 21, dtype, device=gpu_device)
+    pcfg, w = plain.read_model_dir(tmp_path)
+    _, model = load_model(tmp_path, dtype, gpu_device)
+    requests = {"long": random_prompt(777, cfg["vocab_size"], 140)}
+    ref = {rid: plain.forward_logits(pcfg, w, t) for rid, t in requests.items()}
+    rtol, atol = TOL[dtype]
+    runner = runner_for(model, 16, 777 // 16 + 2)
+    drives.compare(drives.drive_whole(runner, requests), ref, rtol, atol)
+    drives.compare(drives.drive_portions(runner, requests, sizes=(477, 300)), ref, rtol, atol)
