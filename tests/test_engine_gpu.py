@@ -264,5 +264,18 @@ def test_long_prompt_through_the_kernels_of_many_rows(dtype, tmp_path, gpu_devic
     ref = {rid: plain.forward_logits(pcfg, w, t) for rid, t in requests.items()}
     rtol, atol = TOL[dtype]
     runner = runner_for(model, 16, 777 // 16 + 2)
-    drives.compare(drives.drive_whole(runner, requests), ref, rtol, atol)
-    drives.compare(drives.drive_portions(runner, requests, sizes=(477, 300)), ref, rtol, atol)
+    ops, called = model.ctx.ops, []
+    call = ops._call
+    ops._call = lambda fn, *args: (called.append(fn.__name__), call(fn, *args))[1]
+    try:
+        drives.compare(drives.drive_whole(runner, requests), ref, rtol, atol)
+        whole = list(called)
+        drives.compare(drives.drive_portions(runner, requests, sizes=(477, 300)), ref, rtol, atol)
+    finally:
+        ops._call = call
+    if dtype == torch.bfloat16:
+        # every product that ends a sub-layer but the model's last, and every one behind
+        # a norm but the first
+        assert whole.count("ts_gemm_tiled_tail_bf16") == 2 * 3 - 1
+        assert whole.count("ts_gemm_tiled_scaled_bf16") == 2 * 3 - 1
+        assert "ts_gemm_tiled_tail_bf16" not in called[len(whole):]
