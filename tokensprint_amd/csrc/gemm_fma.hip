@@ -91,17 +91,68 @@ __global__ __launch_bounds__(256) void gemm_fma_rows_kernel(const TA* __restrict
   for (int m = 0; m < MR; ++m)
 #pragma unroll
     for (int c = 0; c < CPW; ++c) acc[m][c] = 0.f;
-  for (int k = lane * 4; k < K; k += kWave * 4) {
-    f32x4_fma w[CPW];
+  // Few rows (a decode step): the rows of W are read once and come from memory; four
+  // stretches of them are asked for before the first is used, and each again four ahead, so
+  // that a compute unit's few waves keep enough bytes on the way (a decode step's product
+  // has one workgroup a unit; stretch after stretch it ran at a tenth of the memory's
+  // rate).  The rows of A, the same for every wave, come out of the caches one stretch
+  // ahead.  The sums' order is that of the plain loop.
+  if constexpr (MR > 8) {
+    // many rows (a prompt's portion, workgroups enough to hide the waits): stretch after
+    // stretch, a row at a time, so that the sums and not the rows hold the registers
+    for (int k = lane * 4; k < K; k += kWave * 4) {
+      f32x4_fma w[CPW];
 #pragma unroll
-    for (int c = 0; c < CPW; ++c) w[c] = load4_fma(W + min(n0 + c, (int64_t)N - 1) * K + k);
+      for (int c = 0; c < CPW; ++c) w[c] = load4_fma(W + min(n0 + c, (int64_t)N - 1) * K + k);
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      const f32x4_fma a = load4_fma(A + (int64_t)min(m, M - 1) * K + k);
+      for (int m = 0; m < MR; ++m) {
+        const f32x4_fma a = load4_fma(A + (int64_t)min(m, M - 1) * K + k);
 #pragma unroll
-      for (int c = 0; c < CPW; ++c)
+        for (int c = 0; c < CPW; ++c)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[m][c] = fmaf(a[e], w[c][e], acc[m][c]);
+          for (int e = 0; e < 4; ++e) acc[m][c] = fmaf(a[e], w[c][e], acc[m][c]);
+      }
+    }
+  } else {
+    constexpr int kAhead = 4;
+    const int stretches = (K - lane * 4 + kWave * 4 - 1) / (kWave * 4);     // of this lane
+    // (a lane without a stretch i reads the row's last four elements and drops them)
+    auto w_at = [&](int i, int c) {
+      return load4_fma(W + min(n0 + c, (int64_t)N - 1) * K + min(lane * 4 + i * kWave * 4, K - 4));
+    };
+    auto a_at = [&](int i, int m) {
+      return load4_fma(A + (int64_t)min(m, M - 1) * K + min(lane * 4 + i * kWave * 4, K - 4));
+    };
+    f32x4_fma w[kAhead][CPW], a_next[MR];
+#pragma unroll
+    for (int p = 0; p < kAhead; ++p)
+#pragma unroll
+      for (int c = 0; c < CPW; ++c) w[p][c] = w_at(p, c);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) a_next[m] = a_at(0, m);
+    for (int i0 = 0; i0 < stretches; i0 += kAhead) {
+#pragma unroll
+      for (int p = 0; p < kAhead; ++p) {
+        const int i = i0 + p;
+        if (i >= stretches) break;
+        f32x4_fma a[MR];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) a[m] = a_next[m];
+        if (i + 1 < stretches) {
+#pragma unroll
+          for (int m = 0; m < MR; ++m) a_next[m] = a_at(i + 1, m);
+        }
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+          for (int c = 0; c < CPW; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[m][c] = fmaf(a[m][e], w[p][c][e], acc[m][c]);
+        if (i + kAhead < stretches) {
+#pragma unroll
+          for (int c = 0; c < CPW; ++c) w[p][c] = w_at(i + kAhead, c);
+        }
+      }
     }
   }
 #pragma unroll

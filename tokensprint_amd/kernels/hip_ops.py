@@ -11,6 +11,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import Structure, byref, c_float, c_int, c_void_p
 
+import numpy as np
 import torch
 
 from tokensprint_amd.kernels.build import build, find_library
@@ -865,22 +866,23 @@ class HipOps:
         memory (a copy out of pageable memory holds the host until it is done, and the step's
         first attention call, which the GPU is waiting for, makes this list).  Four buffers
         in turn, each free again once its last copy has been made."""
-        host = torch.tensor(rows, dtype=torch.int32)
+        host = np.asarray(rows, dtype=np.int32)
         if self.device.type != "cuda":
-            return host.to(self.device)
+            return torch.from_numpy(host).to(self.device)
         turn = self._staging_turn = (getattr(self, "_staging_turn", -1) + 1) % 4
         if not hasattr(self, "_staging"):
             self._staging = [None] * 4
         slot = self._staging[turn]
-        if slot is None or slot[0].numel() < host.numel():
-            slot = (torch.empty(max(host.numel(), 1 << 14), dtype=torch.int32, pin_memory=True),
+        if slot is None or slot[0].numel() < host.size:
+            slot = (torch.empty(max(host.size, 1 << 14), dtype=torch.int32, pin_memory=True),
                     torch.cuda.Event())
             self._staging[turn] = slot
         else:
             slot[1].synchronize()
-        pinned = slot[0][:host.numel()].view(host.shape)
-        pinned.copy_(host)
-        dev = pinned.to(self.device, non_blocking=True)
+        # (written through numpy: the buffer may have been made under inference mode, which
+        # forbids a tensor's own in-place copy outside it)
+        slot[0].numpy()[:host.size] = host.reshape(-1)
+        dev = slot[0][:host.size].view(host.shape).to(self.device, non_blocking=True)
         slot[1].record()
         return dev
 
