@@ -120,6 +120,7 @@ class HipOps:
         # for the vendor library's algorithms that want scratch memory during a product
         self._library_workspace = torch.empty(64 << 20, dtype=torch.uint8, device=self.device)
         self._timed_plans = False
+        self._staging, self._staging_turn = [None] * 4, -1      # pinned buffers of _upload_ints
         # products of few rows with large weights: ours or the library's, per weight shape
         # (see large_weight_choices)
         self._large_rows, self._large_undecided, self._large_trial = {}, set(), None
@@ -869,9 +870,7 @@ class HipOps:
         host = np.asarray(rows, dtype=np.int32)
         if self.device.type != "cuda":
             return torch.from_numpy(host).to(self.device)
-        turn = self._staging_turn = (getattr(self, "_staging_turn", -1) + 1) % 4
-        if not hasattr(self, "_staging"):
-            self._staging = [None] * 4
+        turn = self._staging_turn = (self._staging_turn + 1) % len(self._staging)
         slot = self._staging[turn]
         if slot is None or slot[0].numel() < host.size:
             slot = (torch.empty(max(host.size, 1 << 14), dtype=torch.int32, pin_memory=True),
