@@ -45,7 +45,7 @@ TINY = {"A": (TINY_A, 0, 4), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 8),
 LAYER_E = qwen3_config(hidden=1024, layers=2, heads=16, kv_heads=8, head_dim=128, inter=3072,
                        vocab=20011, eps=1e-6, theta=1e6, tied=True, max_pos=256)
 # Two layers of the Qwen3-8B and Qwen3-32B shapes: at these widths other routes serve the
-# rows (the library from 9 rows on, the norm as a kernel of its own where the fused form's
+# rows (the library from 16 rows on, the norm as a kernel of its own where the fused form's
 # limits end, key/value groups of 4 and 8 query heads).
 LAYER_F = qwen3_config(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128, inter=12288,
                        vocab=20011, eps=1e-6, theta=1e6, tied=False, max_pos=256)

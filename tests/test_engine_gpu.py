@@ -207,10 +207,10 @@ def wide_bfloat16(request, tmp_path_factory, gpu_device):
 
 
 @pytest.mark.parametrize("captured", [False, True], ids=["eager", "captured"])
-@pytest.mark.parametrize("lanes", [4, 5, 8, 9, 16, 17, 32, 33, 64, 65, 127, 129])
+@pytest.mark.parametrize("lanes", [4, 5, 8, 9, 15, 16, 17, 32, 33, 64, 65, 127, 129])
 def test_decode_lanes_on_both_sides_of_each_kernel_choice(wide_bfloat16, lanes, captured):
     """Which kernel serves a product depends on the number of rows: the output head goes
-    to the library from 5 rows, the layer products of this width from 9, those with a
+    to the library from 5 rows, the layer products of this width from 16, those with a
     short K from 17, everything from 65 (the 8B width, F); at the 0.6B width (E) the layer
     products are this engine's up to 64 rows, with more tiles of rows per workgroup from 17
     and from 33; and from 128 lanes (1,024 tiles of 16 query rows at 8 key/value heads) the

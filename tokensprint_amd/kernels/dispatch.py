@@ -30,9 +30,11 @@ class Dispatch:
     head_columns: int = 16384
     #: weights above `large_weight` elements (the layer shapes of the 8B and 32B models:
     #: products bound by bandwidth, not latency): every workgroup's reading of the rows of
-    #: x costs as much as the weights from 16 rows on and the library is ahead from 9;
-    #: whether it also takes 1 to 8 rows is decided per weight shape by the warm-up
-    library_rows_large: int = 9
+    #: x costs as much as the weights from 16 rows on, and the library is ahead from there
+    #: (a decode step of the 8B shape with 12 requests 4.13 ms here against 4.37 with the
+    #: library, with 16 requests 4.47 against 4.43, with 32 5.59 against 4.92); whether it
+    #: also takes the rows below is decided per weight shape by the warm-up
+    library_rows_large: int = 16
     large_weight: int = 1 << 23
 
     # ---- gate/up product of many rows with the SiLU-multiply in its epilogue: stacked

@@ -343,7 +343,7 @@ class HipOps:
         """Row counts from which products with a large weight may go to the library, for the
         warm-up to try in a captured decode step, the default first; empty unless a large
         weight of a shape that has no choice yet has been met.  At the Qwen3-8B shapes the
-        kernels here are ahead below nine rows (a decode step of one row 3.61 against
+        kernels here are ahead below sixteen rows (a decode step of one row 3.45 against
         4.07 ms), at the 32B shapes (a hidden size of 5,120: 320 or 640 workgroups for 256
         compute units, and a K that the loads' steps divide less well) the library is, by 15
         to 20 %, norm kernels and all.  A choice is kept per weight shape (N, K), so that
