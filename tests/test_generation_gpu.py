@@ -231,10 +231,11 @@ def test_warm_up_chooses_who_multiplies_large_weights(setup, gpu_device, tmp_pat
     L = cfg["max_position_embeddings"]
     engine = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L)
     chosen = dict(ops._large_rows)
-    assert chosen and len(set(chosen.values())) == 1 and set(chosen.values()) <= {9, 1}
+    default = ops.dispatch.library_rows_large
+    assert chosen and len(set(chosen.values())) == 1 and set(chosen.values()) <= {default, 1}
     assert ops.large_weight_choices() == ()          # every shape met has its choice
     assert set(engine.runner.graphs) == set(engine.runner.buckets)     # the trials were dropped
-    for rows in (9, 1):
+    for rows in (default, 1):
         monkeypatch.setattr(ops, "_large_rows", {shape: rows for shape in chosen})
         runner = engine_for(model, d, torch.bfloat16, kvcache_block_size=page, max_model_len=L,
                             warmup=False).runner
