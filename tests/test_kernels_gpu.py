@@ -250,14 +250,16 @@ def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
 @pytest.mark.parametrize("M,N,K,next_n,silu", [(2051, 1024, 2048, 3072, True),
                                                (513, 320, 1024, 400, False),
                                                (700, 576, 4096, 112, True),
-                                               (1030, 1024, 3072, 4096, False)])
+                                               (1030, 1024, 3072, 4096, False),
+                                               (520, 4096, 256, 64, False)])
 def test_gemm_tiled_into_stream(ops, gpu_device, M, N, K, next_n, silu):
     """The tiled product's tail form (adds itself into the float32 stream, hands the stream
     on times the norm's weight, with the rows' sums of squares in slices) and the scaled
     form behind it, each against float32 arithmetic on what it was given, every tile the
     same to the bit; then the two through the provider's entry points against the
     separate product, add-and-norm and product.  The stream's rows differ a hundredfold
-    in size, so that a factor taken from another row shows."""
+    in size, so that a factor taken from another row shows.  (The last case has 128 slices
+    a row: more than the scaled form asks for at a time.)"""
     from tokensprint_amd.kernels.hip_ops import _ptr
     from tokensprint_amd.kernels.stream import NormHint, PreparedRows
     bf = torch.bfloat16
@@ -317,19 +319,22 @@ def test_gemm_tiled_into_stream(ops, gpu_device, M, N, K, next_n, silu):
         torch.testing.assert_close(stream_apart, stream, rtol=1e-2, atol=1e-2)
         # The two round the normed rows to bfloat16 at different places (before or after the
         # division by the root mean square), so each is compared with the exact function of
-        # the stream: a product of N terms of size 0.05 with operands 2^-9 off is 0.01 off
-        # and rounded to 2^-9 of itself, and silu(gate) * up carries both factors' errors.
+        # the stream.  A sum of N products of operands 2^-9 off has noise of about
+        # 2^-9 * sqrt(N) * rms(h) * rms(w) (0.003 at N = 1,024 here); six of those, since
+        # millions of elements are compared, plus the result's own rounding; and
+        # silu(gate) * up carries both factors' noise.
         s64 = stream.double()
         h = s64 * torch.rsqrt((s64 ** 2).mean(1, keepdim=True) + eps) * g.double()
         exact = h @ wn.double().T
+        sigma = 2.0 ** -9 * (N ** 0.5) * float(h.pow(2).mean().sqrt() * wn.double().pow(2).mean().sqrt())
         if silu:
             gate, up = exact[:, :next_n], exact[:, next_n:]
-            exact, slack = gate * torch.sigmoid(gate) * up, 0.02 * (1 + gate.abs() + up.abs())
+            exact, slack = gate * torch.sigmoid(gate) * up, 6 * sigma * (1 + gate.abs() + up.abs())
         else:
-            slack = 0.02
+            slack = 6 * sigma
         for name, got in (("fused", out), ("apart", apart)):
-            excess = (got.double() - exact).abs() - slack - 0.01 * exact.abs()
-            assert excess.max().item() <= 0, f"{name}: {excess.max().item()} beyond the bound"
+            excess = ((got.double() - exact).abs() - slack - 0.01 * exact.abs()).max().item()
+            assert excess <= 0, f"{name}: {excess} beyond the rounding bound"
 
 
 def test_gemm_tiled_refuses_what_it_cannot_take(ops, gpu_device):
