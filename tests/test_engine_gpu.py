@@ -252,8 +252,9 @@ def test_long_prompt_through_the_kernels_of_many_rows(dtype, tmp_path, gpu_devic
     """A prompt of 777 tokens through a small model whose sizes (hidden 320, inner 768:
     multiples of 64 that are no powers of two) the LDS-tiled products take: whole (in
     bfloat16 the products carry the stream's add and the norm from 512 rows on, and the
-    wide attention kernel takes the step) and in portions of 477 and 300 (the separate
-    kernels), both against the plain implementation."""
+    wide attention kernel takes the step), in portions of 477 and 300 (the separate
+    kernels), and in a step of 601 rows that holds most of it beside a short prompt and
+    another request's single token, all against the plain implementation."""
     from helpers import qwen3_config
     cfg = qwen3_config(hidden=320, layers=3, heads=4, kv_heads=2, head_dim=64, inter=768,
                        vocab=1000, eps=1e-6, theta=1e4, tied=True, max_pos=1024)
@@ -279,3 +280,27 @@ def test_long_prompt_through_the_kernels_of_many_rows(dtype, tmp_path, gpu_devic
         assert whole.count("ts_gemm_tiled_tail_bf16") == 2 * 3 - 1
         assert whole.count("ts_gemm_tiled_scaled_bf16") == 2 * 3 - 1
         assert "ts_gemm_tiled_tail_bf16" not in called[len(whole):]
+    # and a step of as many rows made of three requests: most of the long prompt, a short
+    # prompt whole and another request's single token
+    from tokensprint_amd.engine import StepEntry
+    more = {"a": random_prompt(40, cfg["vocab_size"], 141), "b": random_prompt(24, cfg["vocab_size"], 142)}
+    ref.update({rid: plain.forward_logits(pcfg, w, t) for rid, t in more.items()})
+    tokens = dict(requests, **more)
+    runner = runner_for(model, 16, (777 + 40 + 24) // 16 + 4)
+    rc = {rid: runner.manager.admit(rid) for rid in tokens}
+    col = drives.Collector()
+
+    def step(parts):
+        entries = []
+        for rid, lo, hi in parts:
+            runner.manager.extend(rc[rid], hi)
+            entries.append(StepEntry(rc[rid], tokens[rid][lo:hi], lo, list(range(hi - lo))))
+        col.take(entries, runner.step(entries))
+
+    step([("b", 0, 23)])
+    step([("long", 0, 560), ("a", 0, 40), ("b", 23, 24)])
+    step([("long", 560, 777)])
+    for r in rc.values():
+        runner.manager.free(r)
+    runner.manager.check()
+    drives.compare(col, ref, rtol, atol)
