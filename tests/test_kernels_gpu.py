@@ -251,7 +251,8 @@ def test_gemm_tiled_with_silu_mul(ops, gpu_device, M, I, K):
                                                (513, 320, 1024, 400, False),
                                                (700, 576, 4096, 112, True),
                                                (1030, 1024, 3072, 4096, False),
-                                               (520, 4096, 256, 64, False)])
+                                               (520, 4096, 256, 64, False),
+                                               (8200, 1024, 2048, 3072, True)])
 def test_gemm_tiled_into_stream(ops, gpu_device, M, N, K, next_n, silu):
     """The tiled product's tail form (adds itself into the float32 stream, hands the stream
     on times the norm's weight, with the rows' sums of squares in slices) and the scaled
