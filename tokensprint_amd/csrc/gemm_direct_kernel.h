@@ -41,7 +41,7 @@ __global__ __launch_bounds__(WK* kWave) void gemm_direct_kernel(DirectArgs a) {
   // several, and the piece a product needs is moved down to the first rows' lanes (a DPP
   // move; the other rows of the operand only produce results that nobody stores).
   static_assert((CW == 16 || CW == 8 || CW == 4) && (AR == 16 || AR == 8 || AR == 4), "rows");
-  static_assert(CW == 16 || (MT == 1 && !PAIR && !NORM && !SCALED), "narrow tiles: plain and tail form");
+  static_assert(CW == 16 || (MT == 1 && !PAIR && !NORM), "narrow tiles: one tile of rows, one weight, A from memory");
   static_assert(AR == 16 || (MT == 1 && !NORM), "packed rows of A: one tile, A from memory");
   constexpr int GW = 16 / CW, GA = 16 / AR;          // pieces per load instruction
   static_assert(S % GW == 0 && S % GA == 0, "a step holds whole instructions");
